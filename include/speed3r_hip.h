@@ -1,0 +1,128 @@
+/*
+ * speed3r_hip.h -- C ABI of the MI355X (gfx950) implementation of Speed3R's global
+ * top-k block-sparse attention path.
+ *
+ * The reference implements this path in Python + Triton and has no FFI of its own; each
+ * entry point below replaces the Python-level call named in its comment (paths relative to
+ * the reference root).  All tensors are device pointers; strides are in ELEMENTS; the last
+ * (head_dim) stride of every q/k/v/o tensor is 1.  Launches are asynchronous on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream).  Every function returns
+ * S3R_OK or a negative error code and never throws; s3r_last_error() gives the message of
+ * the calling thread's last failure.  Nothing is allocated, no global state is kept.
+ */
+#ifndef SPEED3R_HIP_H
+#define SPEED3R_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of q/k/v/o/gate tensors ("I/O dtype") */
+#define S3R_F32 0
+#define S3R_BF16 1
+#define S3R_F16 2
+
+#define S3R_OK 0
+#define S3R_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, misaligned pointer/stride */
+#define S3R_ERR_UNSUPPORTED (-2) /* shape/dtype outside what the kernels are built for */
+#define S3R_ERR_HIP (-3)         /* a HIP runtime call or launch failed */
+
+/* Library identification, e.g. "speed3r_hip 0.1 gfx950". */
+const char* s3r_version(void);
+/* Message of the calling thread's most recent failing call ("" if none). */
+const char* s3r_last_error(void);
+/* Bit set of optional features built into this library. */
+#define S3R_CAP_FUSED_TOPK 1 /* s3r_compressed_attn_topk selects without a scores buffer */
+int s3r_capabilities(void);
+
+/*
+ * Block mean-pooling: y[b,h,j,:] = mean over tokens [j*block, min((j+1)*block, N)) of x[b,h,t,:].
+ * Replaces F.avg_pool1d(kernel=stride=block) in pi3/models/layers/sparse_attention.py:97-99
+ * (applied there to the packed qkv; pass H = 3*heads with the packed strides to pool all
+ * three at once).  fp32 accumulation, result rounded to `dtype`.  y is [B,H,ceil(N/block),D]
+ * with its own strides.  A ragged tail block is a mean over its valid tokens.
+ * Requires D*sizeof(elt) to be a power-of-two multiple of 16 bytes up to 1024, and 16-byte
+ * aligned pointers/strides.
+ */
+int s3r_pool_mean(const void* x, void* y, int B, int H, int64_t N, int D, int block,
+                  int64_t sxb, int64_t sxh, int64_t sxn,
+                  int64_t syb, int64_t syh, int64_t syn,
+                  int dtype, void* stream);
+
+/*
+ * Compressed-branch attention with top-k block selection.
+ * Replaces flash_attn_topk_func / forward_with_topk / _fwd_kernel_with_topk
+ * (pi3/models/sparse_attn/flash_attention_topk.py:22-200,633-668), non-causal, no bias.
+ *   o[b,h,i,:]   = softmax_j(scale * q[i].k[j]) v[j]          (I/O dtype)
+ *   lse[b,h,i]   = log sum_j exp(scale * q[i].k[j])           (fp32, optional, [B,H,Lq] contiguous)
+ *   topk_idx[b,h,i,0..K-1] = columns of the K largest raw UNSCALED fp32 q[i].k[j], ordered by
+ *       descending 64-bit key (sortable(bits(s)) << 32 | Lk-1-j): descending score, equal
+ *       scores lowest column first; if Lk < K the trailing slots hold Lk-1.
+ *       (int32, optional, [B,H,Lq,K] contiguous)
+ *   scores[b,h,i,j] = raw fp32 q[i].k[j]                      (optional, [B,H,Lq,Lk] contiguous)
+ * When `scores` is given the indices are computed from exactly those stored values, so
+ * s3r_topk_rows() on `scores` reproduces `topk_idx` bit for bit.  When `scores` is NULL the
+ * selection is fused into the attention kernel and the scores never reach HBM.
+ * Requires D <= 64 (D == 64 for the MFMA path), K a power of two <= 64.
+ */
+int s3r_compressed_attn_topk(const void* q, const void* k, const void* v,
+                             void* o, float* lse, int32_t* topk_idx, float* scores,
+                             int B, int H, int Lq, int Lk, int D, int K,
+                             int64_t sqb, int64_t sqh, int64_t sqm,
+                             int64_t skb, int64_t skh, int64_t skn,
+                             int64_t svb, int64_t svh, int64_t svn,
+                             int64_t sob, int64_t soh, int64_t som,
+                             float softmax_scale, int dtype, void* stream);
+
+/*
+ * Row-wise exact top-k of a materialised fp32 score matrix (same ordering rule as above).
+ * Stands for the streaming bitonic top-k inside _fwd_kernel_with_topk
+ * (flash_attention_topk.py:112-132,145-152; topk_utils.py:11-23,438-501).
+ * scores: `rows` rows of `cols` floats, row r at scores + r*row_stride; idx: [rows, K] int32.
+ * 1 <= K <= 64.
+ */
+int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int64_t row_stride,
+                  int K, void* stream);
+
+/*
+ * Selection-branch attention: every `block`-row query block attends to the K key blocks its
+ * index row lists, in list order.
+ * Replaces topk_blocksparse_attention / _topk_blocksparse_attention_fwd /
+ * block_sparse_forward_kernel (pi3/models/sparse_attn/topk_blocksparse_attention.py:35-128,
+ * 852-904,1093-1121).
+ *   idx: int32 [B,H,ceil(N/block),K] (strides sib,sih,sim; last stride 1), block units;
+ *        entries < 0 or with idx*block >= N are skipped; duplicates are attended twice.
+ *   o:   I/O dtype [B,H,N,D];  lse: optional fp32 [B,H,N] contiguous.
+ * Keys beyond N in a partial last block are masked out; a query block with no valid entry
+ * gives zeros.  block in {16,32,64}, D <= 64 (MFMA path: block == 64, D == 64, bf16/fp16).
+ */
+int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx,
+                    void* o, float* lse,
+                    int B, int H, int64_t N, int D, int block, int K,
+                    int64_t sqb, int64_t sqh, int64_t sqn,
+                    int64_t skb, int64_t skh, int64_t skn,
+                    int64_t svb, int64_t svh, int64_t svn,
+                    int64_t sob, int64_t soh, int64_t son,
+                    int64_t sib, int64_t sih, int64_t sim,
+                    float softmax_scale, int dtype, void* stream);
+
+/*
+ * Gated merge of the two branches, written in the [B,N,H*D] layout the output projection
+ * reads:  out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d].
+ * Replaces the einops/broadcast expression in pi3/models/layers/sparse_attention.py:127-136.
+ * Each product and the sum are rounded to the I/O dtype, like the eager expression.
+ * gate strides sgb,sgh,sgn address the pair (last stride 1); out is contiguous.
+ */
+int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void* out,
+                    int B, int H, int64_t N, int D, int block,
+                    int64_t scb, int64_t sch, int64_t scm,
+                    int64_t ssb, int64_t ssh, int64_t ssn,
+                    int64_t sgb, int64_t sgh, int64_t sgn,
+                    int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPEED3R_HIP_H */

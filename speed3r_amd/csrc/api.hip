@@ -1,0 +1,87 @@
+// C-ABI entry points of the two attention operators: argument validation and kernel choice.
+#include "s3r_common.h"
+#include "attn_params.h"
+
+namespace s3r {
+
+char* last_error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+static bool dtype_ok(int dtype) { return dtype == S3R_F32 || dtype == S3R_BF16 || dtype == S3R_F16; }
+
+// 16-byte vector access along head_dim needs aligned bases and row strides
+static bool vec_ok(const void* p, int es, int64_t s0, int64_t s1, int64_t s2) {
+  return aligned16(p) && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0 && (s2 * es) % 16 == 0;
+}
+
+}  // namespace s3r
+
+using namespace s3r;
+
+extern "C" const char* s3r_version(void) { return "speed3r_hip 0.1 gfx950"; }
+
+extern "C" const char* s3r_last_error(void) { return last_error_buffer(); }
+
+extern "C" int s3r_capabilities(void) { return 0; }
+
+extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void* v, void* o, float* lse, int32_t* topk_idx,
+                                        float* scores, int B, int H, int Lq, int Lk, int D, int K,
+                                        int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
+                                        int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t som,
+                                        float softmax_scale, int dtype, void* stream) {
+  if (!q || !k || !v || !o) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: null pointer");
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || D <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: non-positive size");
+  if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: dtype %d", dtype);
+  if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: head_dim %d > 64", D);
+  if (topk_idx != nullptr && (K < 1 || K > 64 || (K & (K - 1)) != 0))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: top-k %d must be a power of two <= 64", K);
+
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.scores = scores; p.idx = nullptr; p.topk_idx = topk_idx;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.D = D; p.block = 64; p.K = K;
+  p.sqb = sqb; p.sqh = sqh; p.sqm = sqm; p.skb = skb; p.skh = skh; p.skn = skn;
+  p.svb = svb; p.svh = svh; p.svn = svn; p.sob = sob; p.soh = soh; p.som = som;
+  p.scale = softmax_scale;
+
+  const int es = elt_size(dtype);
+  const bool mfma_ok = dtype != S3R_F32 && D == 64 && softmax_scale > 0.f && vec_ok(q, es, sqb, sqh, sqm) &&
+                       vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, som);
+  if (mfma_ok) return launch_compressed_mfma(p, dtype, stream);
+  if (topk_idx != nullptr && scores == nullptr)
+    return fail(S3R_ERR_UNSUPPORTED,
+                "s3r_compressed_attn_topk: fused selection needs bf16/fp16, head_dim 64, 16-byte aligned tensors; "
+                "pass a scores buffer for other shapes");
+  int rc = launch_attn_simple(p, dtype, /*select=*/false, stream);
+  if (rc != S3R_OK) return rc;
+  if (topk_idx != nullptr) rc = s3r_topk_rows(scores, topk_idx, (int64_t)B * H * Lq, Lk, Lk, K, stream);
+  return rc;
+}
+
+extern "C" int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx, void* o, float* lse,
+                               int B, int H, int64_t N, int D, int block, int K,
+                               int64_t sqb, int64_t sqh, int64_t sqn, int64_t skb, int64_t skh, int64_t skn,
+                               int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t son,
+                               int64_t sib, int64_t sih, int64_t sim, float softmax_scale, int dtype, void* stream) {
+  if (!q || !k || !v || !idx || !o) return fail(S3R_ERR_BAD_ARG, "s3r_select_attn: null pointer");
+  if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || K <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_select_attn: non-positive size");
+  if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: dtype %d", dtype);
+  if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: head_dim %d > 64", D);
+  if (block != 4 && block != 16 && block != 32 && block != 64)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: block %d not in {4,16,32,64}", block);
+
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.scores = nullptr; p.idx = idx; p.topk_idx = nullptr;
+  p.B = B; p.H = H; p.Lq = N; p.Lk = N; p.D = D; p.block = block; p.K = K;
+  p.sqb = sqb; p.sqh = sqh; p.sqm = sqn; p.skb = skb; p.skh = skh; p.skn = skn;
+  p.svb = svb; p.svh = svh; p.svn = svn; p.sob = sob; p.soh = soh; p.som = son;
+  p.sib = sib; p.sih = sih; p.sim = sim;
+  p.scale = softmax_scale;
+
+  const int es = elt_size(dtype);
+  const bool mfma_ok = dtype != S3R_F32 && D == 64 && block == 64 && softmax_scale > 0.f && vec_ok(q, es, sqb, sqh, sqn) &&
+                       vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, son);
+  if (mfma_ok) return launch_select_mfma(p, dtype, stream);
+  return launch_attn_simple(p, dtype, /*select=*/true, stream);
+}

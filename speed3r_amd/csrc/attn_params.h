@@ -1,0 +1,32 @@
+// Argument block shared by the attention kernels (compressed branch and selection branch).
+#pragma once
+#include <stdint.h>
+
+namespace s3r {
+
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;          // optional [B,H,Lq]
+  float* scores;       // optional [B,H,Lq,Lk], compressed branch only
+  const int32_t* idx;  // selection branch: [B,H,ceil(Lq/block),K]
+  int32_t* topk_idx;   // compressed branch, fused selection: [B,H,Lq,K]
+  int B, H;
+  int64_t Lq, Lk;
+  int D, block, K;
+  int64_t sqb, sqh, sqm;
+  int64_t skb, skh, skn;
+  int64_t svb, svh, svn;
+  int64_t sob, soh, som;
+  int64_t sib, sih, sim;
+  float scale;
+};
+
+// launchers implemented in the .hip files; each returns S3R_OK or an error code
+int launch_attn_simple(const AttnParams& p, int dtype, bool select, void* stream);
+int launch_select_mfma(const AttnParams& p, int dtype, void* stream);
+int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream);
+
+}  // namespace s3r

@@ -1,0 +1,148 @@
+// Block mean-pooling and the gated merge: the two pure HBM-streaming kernels of the path.
+//
+// Both move 16 bytes per lane per access.  Pooling gives one wavefront to one
+// (batch, head, block): the wave's 64 lanes cover 64/LPR token rows per load (LPR = lanes per
+// head_dim row), accumulate in fp32 and fold the row groups with xor-shuffles.  The merge
+// maps consecutive lanes to consecutive 16-byte chunks of the [B,N,H*D] output so stores
+// are fully coalesced, and reads the per-head planes in 128-byte row segments.
+#include "s3r_common.h"
+
+namespace s3r {
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_mean_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int H, int64_t N, int D, int block, int64_t Nc,
+    int64_t total, int64_t sxb, int64_t sxh, int64_t sxn, int64_t syb, int64_t syh, int64_t syn) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= total) return;
+  const int64_t j = w % Nc;
+  const int64_t bh = w / Nc;
+  const int h = (int)(bh % H);
+  const int64_t b = bh / H;
+  const int lpr = D / VEC;   // lanes per row, a power of two <= 64
+  const int rpw = 64 / lpr;  // rows per wave-wide load
+  const int r0 = lane / lpr;
+  const int dc = lane - r0 * lpr;
+  const int64_t t0 = j * block;
+  const int nvalid = (int)((N - t0 < block) ? (N - t0) : block);
+  const T* base = x + b * sxb + h * sxh + t0 * sxn + dc * VEC;
+
+  float acc[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; i++) acc[i] = 0.f;
+#pragma unroll 8
+  for (int r = r0; r < nvalid; r += rpw) {
+    uint4 raw = *reinterpret_cast<const uint4*>(base + (int64_t)r * sxn);
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) acc[i] += to_f32(e[i]);
+  }
+  for (int off = lpr; off < 64; off <<= 1) {
+#pragma unroll
+    for (int i = 0; i < VEC; i++) acc[i] += __shfl_xor(acc[i], off);
+  }
+  if (r0 == 0) {
+    uint4 raw;
+    T* e = reinterpret_cast<T*>(&raw);
+    const float cnt = (float)nvalid;
+#pragma unroll
+    for (int i = 0; i < VEC; i++) e[i] = from_f32<T>(acc[i] / cnt);
+    *reinterpret_cast<uint4*>(y + b * syb + h * syh + j * syn + dc * VEC) = raw;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_merge_kernel(
+    const T* __restrict__ oc, const T* __restrict__ os, const T* __restrict__ gate, T* __restrict__ out,
+    int H, int64_t N, int D, int block, uint32_t per_batch,
+    int64_t scb, int64_t sch, int64_t scm, int64_t ssb, int64_t ssh, int64_t ssn,
+    int64_t sgb, int64_t sgh, int64_t sgn) {
+#pragma clang fp contract(off)  // products and sum stay separately rounded operations
+  constexpr int VEC = 16 / sizeof(T);
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;  // chunk index within the batch entry
+  if (i >= per_batch) return;
+  const int64_t b = blockIdx.y;
+  const uint32_t lpr = (uint32_t)D / VEC;
+  const uint32_t dc = i % lpr;
+  const uint32_t t = i / lpr;
+  const uint32_t h = t % (uint32_t)H;
+  const uint32_t n = t / (uint32_t)H;
+  const T* g = gate + b * sgb + h * sgh + (int64_t)n * sgn;
+  const float g0 = to_f32(g[0]);
+  const float g1 = to_f32(g[1]);
+  uint4 rs = *reinterpret_cast<const uint4*>(os + b * ssb + h * ssh + (int64_t)n * ssn + dc * VEC);
+  uint4 rc = *reinterpret_cast<const uint4*>(oc + b * scb + h * sch + (int64_t)(n / (uint32_t)block) * scm + dc * VEC);
+  const T* es = reinterpret_cast<const T*>(&rs);
+  const T* ec = reinterpret_cast<const T*>(&rc);
+  uint4 ro;
+  T* eo = reinterpret_cast<T*>(&ro);
+#pragma unroll
+  for (int e = 0; e < VEC; e++) {
+    // same rounding points as the eager expression: each product, then the sum
+    const float a = round_to<T>(g0 * to_f32(ec[e]));
+    const float c = round_to<T>(g1 * to_f32(es[e]));
+    eo[e] = from_f32<T>(a + c);
+  }
+  *reinterpret_cast<uint4*>(out + ((int64_t)b * per_batch + i) * VEC) = ro;
+}
+
+}  // namespace s3r
+
+using namespace s3r;
+
+extern "C" int s3r_pool_mean(const void* x, void* y, int B, int H, int64_t N, int D, int block,
+                             int64_t sxb, int64_t sxh, int64_t sxn, int64_t syb, int64_t syh, int64_t syn,
+                             int dtype, void* stream) {
+  if (!x || !y) return fail(S3R_ERR_BAD_ARG, "s3r_pool_mean: null pointer");
+  if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || block <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_pool_mean: non-positive size");
+  if (dtype != S3R_F32 && dtype != S3R_BF16 && dtype != S3R_F16) return fail(S3R_ERR_UNSUPPORTED, "s3r_pool_mean: dtype %d", dtype);
+  const int es = elt_size(dtype);
+  const int vec = 16 / es;
+  const int lpr = D / vec;
+  if (D % vec != 0 || lpr > 64 || (lpr & (lpr - 1)) != 0)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_pool_mean: head_dim %d (row bytes must be a power-of-two multiple of 16, <= 1024)", D);
+  if (!aligned16(x) || !aligned16(y) || (sxb * es) % 16 || (sxh * es) % 16 || (sxn * es) % 16 || (syb * es) % 16 ||
+      (syh * es) % 16 || (syn * es) % 16)
+    return fail(S3R_ERR_BAD_ARG, "s3r_pool_mean: pointers and strides must be 16-byte aligned");
+  const int64_t Nc = (N + block - 1) / block;
+  const int64_t total = (int64_t)B * H * Nc;
+  const int64_t nwg = (total + 3) / 4;
+  if (nwg > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_pool_mean: too many blocks");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)nwg), blk(256);
+  if (dtype == S3R_F32)
+    hipLaunchKernelGGL(pool_mean_kernel<float>, grid, blk, 0, st, (const float*)x, (float*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
+  else if (dtype == S3R_BF16)
+    hipLaunchKernelGGL(pool_mean_kernel<bf16_t>, grid, blk, 0, st, (const bf16_t*)x, (bf16_t*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
+  else
+    hipLaunchKernelGGL(pool_mean_kernel<f16_t>, grid, blk, 0, st, (const f16_t*)x, (f16_t*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
+  return check_launch("s3r_pool_mean");
+}
+
+extern "C" int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void* out,
+                               int B, int H, int64_t N, int D, int block,
+                               int64_t scb, int64_t sch, int64_t scm, int64_t ssb, int64_t ssh, int64_t ssn,
+                               int64_t sgb, int64_t sgh, int64_t sgn, int dtype, void* stream) {
+  if (!o_cmp || !o_sel || !gate || !out) return fail(S3R_ERR_BAD_ARG, "s3r_gated_merge: null pointer");
+  if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || block <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_gated_merge: non-positive size");
+  if (dtype != S3R_F32 && dtype != S3R_BF16 && dtype != S3R_F16) return fail(S3R_ERR_UNSUPPORTED, "s3r_gated_merge: dtype %d", dtype);
+  const int es = elt_size(dtype);
+  const int vec = 16 / es;
+  if (D % vec != 0) return fail(S3R_ERR_UNSUPPORTED, "s3r_gated_merge: head_dim %d not a multiple of %d", D, vec);
+  if (!aligned16(o_cmp) || !aligned16(o_sel) || !aligned16(out) || (scb * es) % 16 || (sch * es) % 16 || (scm * es) % 16 ||
+      (ssb * es) % 16 || (ssh * es) % 16 || (ssn * es) % 16)
+    return fail(S3R_ERR_BAD_ARG, "s3r_gated_merge: o_cmp/o_sel/out pointers and strides must be 16-byte aligned");
+  const int64_t per_batch = N * H * (D / vec);
+  if (per_batch > 0xffffff00LL || B > 65535) return fail(S3R_ERR_UNSUPPORTED, "s3r_gated_merge: tensor too large for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)((per_batch + 255) / 256), (unsigned)B), blk(256);
+  if (dtype == S3R_F32)
+    hipLaunchKernelGGL(gated_merge_kernel<float>, grid, blk, 0, st, (const float*)o_cmp, (const float*)o_sel, (const float*)gate, (float*)out, H, N, D, block, (uint32_t)per_batch, scb, sch, scm, ssb, ssh, ssn, sgb, sgh, sgn);
+  else if (dtype == S3R_BF16)
+    hipLaunchKernelGGL(gated_merge_kernel<bf16_t>, grid, blk, 0, st, (const bf16_t*)o_cmp, (const bf16_t*)o_sel, (const bf16_t*)gate, (bf16_t*)out, H, N, D, block, (uint32_t)per_batch, scb, sch, scm, ssb, ssh, ssn, sgb, sgh, sgn);
+  else
+    hipLaunchKernelGGL(gated_merge_kernel<f16_t>, grid, blk, 0, st, (const f16_t*)o_cmp, (const f16_t*)o_sel, (const f16_t*)gate, (f16_t*)out, H, N, D, block, (uint32_t)per_batch, scb, sch, scm, ssb, ssh, ssn, sgb, sgh, sgn);
+  return check_launch("s3r_gated_merge");
+}

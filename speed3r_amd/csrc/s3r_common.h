@@ -1,0 +1,69 @@
+// Shared host/device helpers for the gfx950 kernels of the sparse global-attention path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/speed3r_hip.h"
+
+namespace s3r {
+
+// ---- error reporting (host) -------------------------------------------------------------------
+char* last_error_buffer();  // thread-local, 512 bytes
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(last_error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(S3R_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return S3R_OK;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int elt_size(int dtype) { return dtype == S3R_F32 ? 4 : 2; }
+
+// ---- element types ----------------------------------------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+// value of x after a round trip through the I/O type (the reference rounds probabilities to
+// the value dtype before the PV product).  The empty asm keeps the compiler from folding the
+// narrowing conversion away when it tracks the value in fp32.
+template <typename T> __device__ __forceinline__ float round_to(float x) {
+  T t = (T)x;
+  unsigned short u = __builtin_bit_cast(unsigned short, t);
+  asm volatile("" : "+v"(u));
+  return (float)__builtin_bit_cast(T, u);
+}
+template <> __device__ __forceinline__ float round_to<float>(float x) { return x; }
+
+// fp32 bit pattern -> order-preserving u32: negative values flip all bits, others the sign bit.
+__device__ __forceinline__ uint32_t sortable_key(float s) {
+  uint32_t b = __float_as_uint(s);
+  return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
+}
+
+constexpr int kWave = 64;
+
+}  // namespace s3r

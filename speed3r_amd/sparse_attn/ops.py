@@ -1,0 +1,208 @@
+"""Torch-facing wrappers of the C-ABI entry points.
+
+PyTorch supplies device memory and the current HIP stream; the arithmetic is done by the
+hand-written gfx950 kernels behind ``include/speed3r_hip.h``.  Every function takes and
+returns HIP-device tensors and raises if the library is not built -- there is no CPU or
+eager fallback.
+
+Layouts follow the reference operators: q/k/v/o are ``[B, H, L, D]`` with a contiguous last
+dimension; indices are int32 ``[B, H, n_query_blocks, K]`` in block units.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.S3R_F32, torch.bfloat16: _lib.S3R_BF16, torch.float16: _lib.S3R_F16}
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, bfloat16 or float16") from None
+
+
+def _need_device(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError("speed3r_amd operators run on HIP device tensors only (got a CPU tensor)")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _last_contig(t: torch.Tensor) -> torch.Tensor:
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _forward_only(*ts: torch.Tensor) -> None:
+    if torch.is_grad_enabled() and any(t.requires_grad for t in ts):
+        raise RuntimeError("speed3r_amd operators are forward-only; call them under torch.no_grad()")
+
+
+def pool_mean(x: torch.Tensor, block: int) -> torch.Tensor:
+    """Mean over non-overlapping runs of ``block`` tokens: [B,H,N,D] -> [B,H,ceil(N/block),D].
+
+    ``x`` may be any strided view with a contiguous last dimension (e.g. a head-major view of
+    the packed qkv projection).  A ragged tail block is a mean over its valid tokens.
+    """
+    _need_device(x)
+    _forward_only(x)
+    x = _last_contig(x)
+    b, h, n, d = x.shape
+    nc = -(-n // block)
+    y = torch.empty((b, h, nc, d), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().s3r_pool_mean(x.data_ptr(), y.data_ptr(), b, h, n, d, block,
+                                      x.stride(0), x.stride(1), x.stride(2),
+                                      y.stride(0), y.stride(1), y.stride(2), _code(x), _stream(x))
+    _lib.check(rc, "s3r_pool_mean")
+    return y
+
+
+def pool_qkv_packed(qkv: torch.Tensor, num_heads: int, block: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Pool the packed projection ``[B, N, 3*H*D]`` (layout ``(qkv h d)``) in one launch.
+
+    Returns pooled q, k, v as ``[B, H, Nc, D]`` views of one ``[B, 3H, Nc, D]`` buffer.
+    """
+    b, n, c3 = qkv.shape
+    d = c3 // (3 * num_heads)
+    view = qkv.view(b, n, 3 * num_heads, d).permute(0, 2, 1, 3)  # [B, 3H, N, D], strided
+    y = pool_mean(view, block)
+    return y[:, :num_heads], y[:, num_heads:2 * num_heads], y[:, 2 * num_heads:]
+
+
+def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk: Optional[int],
+                         softmax_scale: Optional[float] = None, return_scores: bool = False,
+                         return_lse: bool = False, materialize_scores: Optional[bool] = None):
+    """Dense attention over pooled tokens plus, if ``topk`` is given, the top-k columns of the
+    raw scores per query row.
+
+    Returns ``(o, idx)`` with optional ``scores`` ([B,H,Lq,Lk] fp32) and ``lse`` appended when
+    requested.  ``materialize_scores`` forces (True) or forbids (False) the score buffer; by
+    default it is used only when asked for or when the fused selection does not cover the shape.
+    """
+    _need_device(q, k, v)
+    _forward_only(q, k, v)
+    q, k, v = (_last_contig(t) for t in (q, k, v))
+    assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
+    b, h, lq, d = q.shape
+    lk = k.shape[2]
+    assert k.shape == (b, h, lk, d) and v.shape == (b, h, lk, d), "k/v shape mismatch"
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    o = torch.empty_like(q, memory_format=torch.contiguous_format)
+    idx = torch.empty((b, h, lq, topk), dtype=torch.int32, device=q.device) if topk else None
+    fused_ok = q.dtype != torch.float32 and d == 64 and _lib.lib_has_fused_topk()
+    want_scores = return_scores or (materialize_scores is True) or (topk and materialize_scores is None and not fused_ok)
+    if materialize_scores is False and topk and not fused_ok:
+        raise RuntimeError("fused top-k is not available for this dtype/shape; allow a score buffer")
+    scores = torch.empty((b, h, lq, lk), dtype=torch.float32, device=q.device) if want_scores else None
+    lse = torch.empty((b, h, lq), dtype=torch.float32, device=q.device) if return_lse else None
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().s3r_compressed_attn_topk(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+            lse.data_ptr() if lse is not None else None,
+            idx.data_ptr() if idx is not None else None,
+            scores.data_ptr() if scores is not None else None,
+            b, h, lq, lk, d, topk or 0,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            scale, _code(q), _stream(q))
+    _lib.check(rc, "s3r_compressed_attn_topk")
+    out = [o, idx]
+    if return_scores:
+        out.append(scores)
+    if return_lse:
+        out.append(lse)
+    return tuple(out)
+
+
+def topk_rows(scores: torch.Tensor, k: int) -> torch.Tensor:
+    """Exact top-k columns of each row of an fp32 matrix ``[..., rows, cols]`` -> int32 ``[..., rows, k]``.
+
+    Order: descending score, equal scores lowest column first, +0.0 above -0.0; if
+    ``cols < k`` the trailing slots hold ``cols - 1``.
+    """
+    _need_device(scores)
+    assert scores.dtype == torch.float32, "scores must be float32"
+    scores = scores.contiguous()
+    cols = scores.shape[-1]
+    rows = scores.numel() // cols
+    idx = torch.empty((*scores.shape[:-1], k), dtype=torch.int32, device=scores.device)
+    with torch.cuda.device(scores.device):
+        rc = _lib.lib().s3r_topk_rows(scores.data_ptr(), idx.data_ptr(), rows, cols, cols, k, _stream(scores))
+    _lib.check(rc, "s3r_topk_rows")
+    return idx
+
+
+def select_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, block: int,
+                softmax_scale: Optional[float] = None, return_lse: bool = False):
+    """Attention of each ``block``-row query block over the key blocks listed in ``idx``."""
+    _need_device(q, k, v, idx)
+    _forward_only(q, k, v)
+    q, k, v, idx = (_last_contig(t) for t in (q, k, v, idx))
+    assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
+    assert idx.dtype == torch.int32, "topk_idx must be int32"
+    b, h, n, d = q.shape
+    assert k.shape == q.shape and v.shape == q.shape, "q, k, v must share a shape"
+    nqb = -(-n // block)
+    assert idx.shape[:3] == (b, h, nqb), f"topk_idx shape {tuple(idx.shape)} does not match {(b, h, nqb, 'K')}"
+    kk = idx.shape[3]
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    o = torch.empty_like(q, memory_format=torch.contiguous_format)
+    lse = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if return_lse else None
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().s3r_select_attn(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), idx.data_ptr(), o.data_ptr(),
+            lse.data_ptr() if lse is not None else None,
+            b, h, n, d, block, kk,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            idx.stride(0), idx.stride(1), idx.stride(2), scale, _code(q), _stream(q))
+    _lib.check(rc, "s3r_select_attn")
+    return (o, lse) if return_lse else o
+
+
+def gated_merge(o_cmp: torch.Tensor, o_sel: torch.Tensor, gate: torch.Tensor, block: int) -> torch.Tensor:
+    """``out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n//block,d] + gate[b,h,n,1]*o_sel[b,h,n,d]`` -> [B,N,H*D].
+
+    ``gate`` is ``[B,H,N,2]`` in any strided form with a contiguous pair (the reference's
+    ``'b n (h g) -> b h n g'`` view of the gate projection qualifies).
+    """
+    _need_device(o_cmp, o_sel, gate)
+    _forward_only(o_cmp, o_sel, gate)
+    o_cmp, o_sel, gate = (_last_contig(t) for t in (o_cmp, o_sel, gate))
+    assert o_cmp.dtype == o_sel.dtype == gate.dtype, "o_cmp, o_sel, gate must share a dtype"
+    b, h, n, d = o_sel.shape
+    nc = -(-n // block)
+    assert o_cmp.shape == (b, h, nc, d), f"o_cmp shape {tuple(o_cmp.shape)} != {(b, h, nc, d)}"
+    assert gate.shape == (b, h, n, 2), f"gate shape {tuple(gate.shape)} != {(b, h, n, 2)}"
+    out = torch.empty((b, n, h * d), dtype=o_sel.dtype, device=o_sel.device)
+    with torch.cuda.device(o_sel.device):
+        rc = _lib.lib().s3r_gated_merge(
+            o_cmp.data_ptr(), o_sel.data_ptr(), gate.data_ptr(), out.data_ptr(), b, h, n, d, block,
+            o_cmp.stride(0), o_cmp.stride(1), o_cmp.stride(2), o_sel.stride(0), o_sel.stride(1), o_sel.stride(2),
+            gate.stride(0), gate.stride(1), gate.stride(2), _code(o_sel), _stream(o_sel))
+    _lib.check(rc, "s3r_gated_merge")
+    return out
+
+
+def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
+                            block: int = 64, topk: int = 16, softmax_scale: Optional[float] = None,
+                            return_parts: bool = False, materialize_scores: Optional[bool] = None):
+    """The whole path on post-norm/RoPE q, k, v ``[B,H,N,D]`` and gate ``[B,H,N,2]``:
+    pool -> compressed attention + top-k -> selection attention -> gated merge -> ``[B,N,H*D]``.
+    """
+    qc, kc, vc = pool_mean(q, block), pool_mean(k, block), pool_mean(v, block)
+    o_cmp, idx = compressed_attn_topk(qc, kc, vc, topk, softmax_scale, materialize_scores=materialize_scores)
+    o_sel = select_attn(q, k, v, idx, block, softmax_scale)
+    out = gated_merge(o_cmp, o_sel, gate, block)
+    if return_parts:
+        return out, dict(idx=idx, o_cmp=o_cmp, o_sel=o_sel, qc=qc, kc=kc, vc=vc)
+    return out

@@ -1,0 +1,181 @@
+"""Parity of each HIP kernel against the CPU oracle, through the C-ABI (needs an MI355X).
+
+Bars: integer/index results bit-exact; floating point within 2e-2 max-abs for bf16/fp16 I/O and
+1e-5 for fp32 I/O of the oracle evaluated in fp32 on the same (already rounded) inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import speed3r_amd as s3r
+from helpers import from_bf16_bits, max_abs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def _randn(shape, seed, dtype, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _ulp_close(got, want_f32, dtype):
+    """|got - want| within one rounding step of dtype (want given in fp32)."""
+    rel = {torch.float32: 2e-6, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}[dtype]
+    err = (got.float().cpu() - want_f32).abs()
+    return bool((err <= rel * want_f32.abs() + 1e-6).all())
+
+
+# ------------------------------------------------------------------------------------ pooling
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("n,block,d", [(256, 64, 64), (200, 64, 64), (1041, 64, 64), (96, 16, 64), (130, 32, 32), (7, 64, 64)])
+def test_pool_matches_oracle(dtype, n, block, d):
+    x = _randn((2, 3, n, d), n + d, dtype)
+    got = s3r.pool_mean(x.to(DEV), block)
+    assert got.shape == (2, 3, -(-n // block), d) and got.dtype == dtype
+    assert _ulp_close(got, oracle.pool_mean(x, block, out_dtype=torch.float32), dtype)
+
+
+def test_pool_fixture_and_packed_qkv_view(golden):
+    H, N, D = 2, 200, 64
+    q, k, v = (from_bf16_bits(golden[n]) for n in ("q", "k", "v"))
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        got = s3r.pool_mean(t.to(DEV), 64)
+        assert _ulp_close(got, torch.from_numpy(golden[f"pooled_{name}"]), torch.bfloat16)
+    # the layer's packed projection [B, N, (qkv h d)] pooled in one launch through strides
+    packed = torch.stack([q, k, v], dim=0)[:, 0].permute(2, 0, 1, 3).reshape(1, N, 3 * H * D).contiguous()
+    qc, kc, vc = s3r.pool_qkv_packed(packed.to(DEV), H, 64)
+    for name, got in (("q", qc), ("k", kc), ("v", vc)):
+        assert _ulp_close(got, torch.from_numpy(golden[f"pooled_{name}"]), torch.bfloat16)
+
+
+# ------------------------------------------------------------------------------------ merge
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("n,block", [(256, 64), (200, 64), (96, 16)])
+def test_merge_bit_exact(dtype, n, block):
+    b, h, d = 2, 4, 64
+    o_sel = _randn((b, h, n, d), 1, dtype)
+    o_cmp = _randn((b, h, -(-n // block), d), 2, dtype)
+    gate_lin = torch.sigmoid(_randn((b, n, 2 * h), 3, torch.float32)).to(dtype)
+    gate = gate_lin.view(b, n, h, 2).permute(0, 2, 1, 3)          # the reference's strided 'b n (h g) -> b h n g' view
+    got = s3r.gated_merge(o_cmp.to(DEV), o_sel.to(DEV), gate_lin.to(DEV).view(b, n, h, 2).permute(0, 2, 1, 3), block)
+    want = oracle.gated_merge(o_cmp, o_sel, gate, block)
+    assert got.shape == (b, n, h * d)
+    assert torch.equal(got.cpu(), want)
+
+
+def test_merge_fixture(golden):
+    o_cmp, o_sel, gate, want = (from_bf16_bits(golden[n]) for n in ("merge_o_cmp", "merge_o_sel", "gate", "merge_out"))
+    got = s3r.gated_merge(o_cmp.to(DEV), o_sel.to(DEV), gate.to(DEV), 64)
+    assert torch.equal(got.cpu(), want)
+
+
+# ------------------------------------------------------------------------------------ top-k
+@pytest.mark.parametrize("name", ["smooth", "ties", "zeros", "short"])
+def test_topk_fixture_bit_exact(golden, name):
+    scores = torch.from_numpy(golden[f"topk_{name}_scores"])
+    want = golden[f"topk_{name}_idx"]
+    got = s3r.topk_rows(scores.to(DEV), want.shape[1])
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("cols", [1, 5, 63, 64, 65, 131, 1041, 4164])
+@pytest.mark.parametrize("k", [1, 8, 16, 32, 64])
+def test_topk_random_and_tie_heavy_bit_exact(cols, k):
+    rng = np.random.default_rng(cols * 131 + k)
+    smooth = rng.standard_normal((37, cols)).astype(np.float32)
+    ties = rng.integers(-2, 3, size=(37, cols)).astype(np.float32)
+    ties[ties == 0] = np.where(rng.random(np.count_nonzero(ties == 0)) < 0.5, 0.0, -0.0)   # signed zeros mixed in
+    for s in (smooth, ties):
+        got = s3r.topk_rows(torch.from_numpy(s).to(DEV), k).cpu().numpy()
+        np.testing.assert_array_equal(got, oracle.topk_from_scores(s, k))
+
+
+def test_topk_special_values_bit_exact():
+    s = np.array([[1.0, np.inf, np.nan, 2.0, -np.inf, -0.0, 0.0, -np.nan]], dtype=np.float32)
+    got = s3r.topk_rows(torch.from_numpy(s).to(DEV), 8).cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.topk_from_scores(s, 8))
+
+
+# ------------------------------------------------------------------------------------ compressed branch
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("lq,lk", [(150, 150), (131, 131), (64, 64), (1, 1), (100, 300), (300, 100), (1041, 1041)])
+def test_compressed_matches_oracle(dtype, lq, lk):
+    h, d, k = 3, 64, 16
+    q = _randn((1, h, lq, d), lq, dtype, 0.5)
+    kk = _randn((1, h, lk, d), lk + 1, dtype, 0.5)
+    v = _randn((1, h, lk, d), lk + 2, dtype)
+    o, idx, scores, lse = s3r.compressed_attn_topk(q.to(DEV), kk.to(DEV), v.to(DEV), k, return_scores=True, return_lse=True)
+    o_ref, lse_ref, s_ref = oracle.compressed_attention(q, kk, v, out_dtype=torch.float32)
+    assert max_abs(o, o_ref) <= TOL[dtype]
+    assert max_abs(lse, lse_ref) <= 1e-4
+    assert max_abs(scores, s_ref) <= 1e-4                           # same products, different summation order
+    # indices are exact for the scores the kernel produced
+    np.testing.assert_array_equal(idx.cpu().numpy(), oracle.topk_from_scores(scores.cpu(), k))
+
+
+def test_compressed_fixture(golden):
+    qc, kc, vc = (from_bf16_bits(golden[n]) for n in ("qc", "kc", "vc"))
+    o, idx, scores = s3r.compressed_attn_topk(qc.to(DEV), kc.to(DEV), vc.to(DEV), 8, return_scores=True)
+    assert max_abs(o, torch.from_numpy(golden["cmp_out"])) <= 2e-2
+    assert max_abs(scores, torch.from_numpy(golden["cmp_scores"])) <= 1e-4
+
+
+def test_flash_attn_topk_func_signature():
+    q = _randn((1, 2, 200, 64), 5, torch.bfloat16, 0.5)
+    o, idx = s3r.flash_attn_topk_func(q.to(DEV), q.to(DEV), q.to(DEV), 16)
+    assert o.shape == q.shape and o.dtype == q.dtype
+    assert idx.shape == (1, 2, 200, 16) and idx.dtype == torch.int32
+    assert (idx[..., 0].cpu() == torch.arange(200)).float().mean() > 0.95     # q.q is (almost always) the row maximum
+    with pytest.raises(NotImplementedError):
+        s3r.flash_attn_topk_func(q.to(DEV), q.to(DEV), q.to(DEV), 16, None, True)
+
+
+# ------------------------------------------------------------------------------------ selection branch
+def _rand_idx(h, nc, k, seed, with_invalid=True):
+    g = torch.Generator().manual_seed(seed)
+    lo, hi = (-1, nc + 1) if with_invalid else (0, nc)
+    idx = torch.randint(lo, hi, (1, h, nc, k), generator=g, dtype=torch.int32)
+    idx[..., 0] = torch.randint(0, nc, (1, h, nc), generator=g, dtype=torch.int32)
+    return idx
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("n,block,k", [(256, 64, 4), (200, 64, 3), (1041, 64, 16), (2112, 64, 8), (96, 16, 4), (100, 32, 2), (40, 4, 3)])
+def test_select_matches_oracle(dtype, n, block, k):
+    h = 3
+    q = _randn((1, h, n, 64), n, dtype, 0.5)
+    kk = _randn((1, h, n, 64), n + 1, dtype, 0.5)
+    v = _randn((1, h, n, 64), n + 2, dtype)
+    idx = _rand_idx(h, -(-n // block), k, n)
+    o, lse = s3r.select_attn(q.to(DEV), kk.to(DEV), v.to(DEV), idx.to(DEV), block, return_lse=True)
+    o_ref, lse_ref = oracle.select_attention(q, kk, v, idx, block, out_dtype=torch.float32, return_lse=True)
+    assert o.dtype == dtype and o.shape == q.shape
+    assert max_abs(o, o_ref) <= TOL[dtype]
+    assert max_abs(lse, lse_ref) <= 1e-4
+
+
+def test_select_fixture(golden):
+    q, k, v = (from_bf16_bits(golden[n]) for n in ("q", "k", "v"))
+    idx = torch.from_numpy(golden["sel_idx"])
+    o = s3r.topk_blocksparse_attention(q.to(DEV), k.to(DEV), v.to(DEV), idx.to(DEV), 64)
+    assert max_abs(o, torch.from_numpy(golden["sel_out"])) <= 2e-2
+
+
+def test_select_empty_row_gives_zeros_and_strided_inputs_work():
+    n, h = 256, 2
+    qkv = _randn((1, n, 3, h, 64), 9, torch.bfloat16, 0.5).to(DEV)
+    q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))        # [1,h,n,64] strided views of a packed buffer
+    idx = torch.tensor([[-1, -1], [0, 1], [2, 2], [3, 9]], dtype=torch.int32).view(1, 1, 4, 2).expand(1, h, 4, 2).contiguous()
+    o = s3r.select_attn(q, k, v, idx.to(DEV), 64)
+    assert torch.count_nonzero(o[:, :, :64]) == 0
+    o_ref = oracle.select_attention(q.cpu(), k.cpu(), v.cpu(), idx, 64, out_dtype=torch.float32)
+    assert max_abs(o, o_ref) <= 2e-2
+
+
+def test_forward_only_guard():
+    x = torch.zeros((1, 1, 64, 64), dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        s3r.pool_mean(x, 64)
