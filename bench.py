@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse global-attention layer path on one MI355X.
+
+A step is one pass of the hot path (pool q,k,v -> compressed attention + top-k -> selection
+attention -> gated merge) over one synthetic layer input already resident in HBM.  The default
+workload is the headline configuration: 256 frames x 1041 tokens = 266 496 tokens, 16 heads x 64,
+block 64, top-k 16, bf16, seeded low-rank-plus-noise q/k/v.
+
+Prints ONE JSON line: ms/layer as `value`, effective TFLOP/s, per-kernel times measured with HIP
+events on the launch stream, the roofline of the dominant (selection) kernel from its algorithmic
+FLOPs, and a CPU baseline (the Python oracle timed on this host's cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--topk", type=int, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-heads", type=int, default=1, help="heads of the workload the CPU baseline runs")
+    ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
+    return ap.parse_args()
+
+
+def cpu_baseline(q, k, v, gate, block, topk, heads):
+    """Times the oracle (eager fp32 PyTorch + numpy top-k) on `heads` heads of the workload."""
+    import torch
+
+    import oracle
+
+    hs = slice(0, heads)
+    qs, ks, vs, gs = (t[:, hs].float() for t in (q, k, v, gate))
+    t0 = time.perf_counter()
+    oracle.sparse_global_attention(qs, ks, vs, gs, block, topk)
+    dt = time.perf_counter() - t0
+    total_heads = q.shape[1]
+    return {
+        "value": dt * 1e3 * total_heads / heads,
+        "unit": "ms",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle (eager fp32 PyTorch + numpy top-k) on heads 0..{heads - 1} of {total_heads}, all tokens: "
+                  f"{dt:.2f} s measured, scaled x{total_heads // heads} to the full layer",
+    }
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path shards by head "
+              "without collectives, see DESIGN.md", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import speed3r_amd as s3r
+    from speed3r_amd import workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    dev = torch.device("cuda:0")
+    cfg, q, k, v, gate = workloads.make_config(args.config)
+    topk = args.topk or cfg.topk
+    block = workloads.BLOCK
+    n = cfg.tokens
+    qd, kd, vd, gd = (t.to(dev) for t in (q, k, v, gate))
+    mat = True if args.materialize_scores else None
+
+    names = ["pool", "compressed_topk", "select", "merge"]
+
+    def step(events=None):
+        def mark(i):
+            if events is not None:
+                events[i].record()
+        mark(0)
+        qc, kc, vc = s3r.pool_mean(qd, block), s3r.pool_mean(kd, block), s3r.pool_mean(vd, block)
+        mark(1)
+        o_cmp, idx = s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat)
+        mark(2)
+        o_sel = s3r.select_attn(qd, kd, vd, idx, block)
+        mark(3)
+        out = s3r.gated_merge(o_cmp, o_sel, gd, block)
+        mark(4)
+        return out
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(evs[i])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        peak_mem = torch.cuda.max_memory_allocated()
+
+    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
+    f_sel = workloads.selection_flops(n, topk)
+    f_cmp = workloads.compressed_flops(n)
+    sel_tflops = f_sel / (kern_ms["select"] * 1e-3) / 1e12
+    es = 2 if cfg.dtype != torch.float32 else 4
+    nc = -(-n // block)
+    pool_bytes = 3 * (n + nc) * 16 * 64 * es
+    merge_bytes = (2 * n * 16 * 64 + n * 16 * 2 + nc * 16 * 64) * es
+
+    result = {
+        "metric": "ms/layer, global sparse attn @%d frames %s" % (cfg.frames, "bf16" if es == 2 else "fp32"),
+        "value": ms_per_step,
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if es == 2 else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{cfg.name}: {cfg.frames} frames x {workloads.TOKENS_PER_FRAME} tokens = {n} tokens, "
+                        f"16 heads x 64, block {block}, top-k {topk}, B=1",
+            "tokens": n, "heads": 16, "head_dim": 64, "block": block, "topk": topk,
+            "scores": "materialized" if (args.materialize_scores or not s3r._lib.lib_has_fused_topk()) else "fused",
+        },
+        "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
+        "kernels_ms": kern_ms,
+        "hbm_gbs": {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9, "merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9},
+        "peak_mem_gb": peak_mem / 1e9,
+        "roofline": {
+            "kernel": "select_mfma_kernel",
+            "bound": "mfma",
+            "achieved": sel_tflops,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": sel_tflops / PEAK_BF16_TFLOPS,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v, gate, block, topk, args.cpu_heads)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
