@@ -1,12 +1,14 @@
 // Selection-branch attention on the gfx950 matrix cores (bf16 / fp16 I/O, block 64, head_dim 64).
 //
-// One wavefront owns one 64-row query block of one head and walks that block's K selected
-// key blocks; the four waves of a workgroup take four consecutive query blocks and never
+// One wavefront owns one 64-row query block of one head and walks that block's selected key
+// blocks; the four waves of a workgroup take four consecutive query blocks and never
 // synchronise with each other (each has a private LDS region).
 //
 // Data flow per selected key block (64 keys x 64 head_dim):
 //   * the K tile goes global -> registers directly in the MFMA A-operand layout
-//     (lane = key row, 8 consecutive head_dim values = one 16-byte load);
+//     (lane = key row, 8 consecutive head_dim values = one 16-byte load); the loads of the
+//     next tile are issued as soon as the S^T MFMAs of the current one have consumed the
+//     registers, so they fly during the softmax and PV phases;
 //   * S^T = K Q^T with v_mfma_f32_32x32x16: the accumulator layout then puts one QUERY per
 //     lane (column = lane & 31) and 16 keys per 32x32 tile in its registers, so row max / row
 //     sum are in-lane loops plus one exchange with lane ^ 32, and the online-softmax rescale
@@ -14,10 +16,16 @@
 //   * P is rounded to the I/O dtype in registers; the accumulator layout of S^T is already the
 //     B-operand layout of O^T = V^T P^T (contraction index = key), with a fixed permutation of
 //     keys inside each group of 16 that the V operand simply follows;
-//   * the V tile goes global -> LDS row-major and comes back through ds_read_b64_tr_b16, which
-//     hands each lane 4 consecutive KEYS of one head_dim column: the A operand V^T without any
-//     explicit transpose.
+//   * the V tile goes global -> LDS without passing through registers (global_load_lds, 16
+//     bytes per lane, issued right after the previous tile's PV phase has read the buffer, so
+//     it flies during the next S^T and softmax phases) and comes back through
+//     ds_read_b64_tr_b16, which hands each lane 4 consecutive KEYS of one head_dim column: the
+//     A operand V^T without any explicit transpose.  Rows are 128 bytes; the 16-byte chunks
+//     of rows 2,3 (mod 4) are stored with their halves swapped so that the four rows one
+//     transposed read touches fall into four disjoint bank groups.
 // The softmax runs in base 2 on logits pre-multiplied by scale*log2(e); statistics are fp32.
+// The running maximum is only raised when it grows by more than 8 (a factor 256), so the
+// accumulator rescale is skipped for most tiles; the final normalisation makes this exact.
 //
 // Workgroup -> work mapping is XCD-aware: hardware deals workgroups round-robin over the 8
 // XCDs, so workgroup w is given work item (w % 8) * per_xcd + w / 8: each XCD then walks a
@@ -56,12 +64,13 @@ __device__ __forceinline__ float xhalf_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-constexpr int kVLd = 72;  // LDS row stride of the V tile in elements (144 bytes)
+constexpr float kRescaleSlack = 8.0f;  // log2 units the running max may lag behind before a rescale
+constexpr int kVTile = 64 * 64;        // elements of one V tile in LDS (rows of 128 bytes, no padding)
 
 template <typename E>
 __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
   typedef typename MfmaT<E>::V8 V8;
-  __shared__ __attribute__((aligned(16))) E vlds_all[4][64 * kVLd];
+  __shared__ __attribute__((aligned(1024))) E vlds_all[4][kVTile];
 
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -85,8 +94,31 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
   const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
   const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
   const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
+  E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
   const int32_t* idx_row = p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
-  E* vl = vlds_all[wave];
+  E* vl = &vlds_all[wave][0];
+
+  // The block's index list, one entry per lane (K <= 64), compacted to the valid entries in order.
+  const int32_t my_idx = lane < p.K ? idx_row[lane] : -1;
+  uint64_t todo = __ballot(my_idx >= 0 && (int64_t)my_idx * 64 < N);
+  int remaining = __popcll(todo);
+  if (remaining == 0) {  // nothing to attend to: zeros
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      const int64_t row = q0 + qt * 32 + c;
+      if (row < N) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<uint4*>(op + row * p.som + hh * 32 + i * 8) = make_uint4(0, 0, 0, 0);
+        if (p.lse != nullptr && hh == 0) p.lse[((int64_t)b * p.H + h) * N + row] = -INFINITY;
+      }
+    }
+    return;
+  }
+  auto next_start = [&]() -> int64_t {
+    const int t = __ffsll((unsigned long long)todo) - 1;
+    todo &= todo - 1;
+    return (int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64;
+  };
 
   // Q block as the B operand of S^T = K Q^T: lane holds Q[q0 + qt*32 + c][ks*16 + hh*8 .. +8]
   V8 bq[2][4];
@@ -109,48 +141,69 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) ot[dt][qt][r] = 0.f;
-  float m_i[2] = {-INFINITY, -INFINITY};
-  float l_i[2] = {0.f, 0.f};  // per-lane partial row sums (this half's keys)
+  float m_i[2] = {-INFINITY, -INFINITY};  // reference maximum in use (base-2 scaled logits)
+  float l_i[2] = {0.f, 0.f};              // per-lane partial row sums (this half's keys)
   const float sl2 = p.scale * 1.4426950408889634f;
 
-  // per-lane constant parts of the transposed V read addresses
-  const int tr_row = 4 * hh + ((lane & 15) >> 2);
-  const int tr_col = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-
-  for (int t = 0; t < p.K; t++) {
-    const int32_t j = __builtin_amdgcn_readfirstlane(idx_row[t]);
-    const int64_t start = (int64_t)j * 64;
-    if (j < 0 || start >= N) continue;
-    const bool partial = start + 64 > N;
-
-    // K tile: A operand, lane holds K[start + kt*32 + c][ks*16 + hh*8 .. +8]
-    V8 ak[2][4];
+  // K tile: A operand, lane holds K[start + kt*32 + c][ks*16 + hh*8 .. +8].  Addresses are a wave-uniform
+  // 64-bit tile base plus a 32-bit per-lane offset.  Rows beyond N (ragged last block) re-read row N-1: their
+  // scores are masked, and their V rows are zeroed in LDS before use.
+  const uint32_t koff0 = (uint32_t)c * (uint32_t)p.skn + hh * 8;
+  const uint32_t koff1 = (uint32_t)(32 + c) * (uint32_t)p.skn + hh * 8;
+  auto load_k = [&](V8 (&ak)[2][4], int64_t start) {
+    const E* kb = kp + start * p.skn;
+    uint32_t off[2] = {koff0, koff1};
+    if (start + 64 > N) {
+      const uint32_t last = (uint32_t)(N - 1 - start);
+      off[0] = (c < last ? c : last) * (uint32_t)p.skn + hh * 8;
+      off[1] = (32 + c < last ? 32 + c : last) * (uint32_t)p.skn + hh * 8;
+    }
 #pragma unroll
     for (int kt = 0; kt < 2; kt++) {
-      const int64_t row = start + kt * 32 + c;
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
         Frag16B f;
-        f.u = make_uint4(0, 0, 0, 0);
-        if (!partial || row < N) f.u = *reinterpret_cast<const uint4*>(kp + row * p.skn + ks * 16 + hh * 8);
+        f.u = *reinterpret_cast<const uint4*>(kb + off[kt] + ks * 16);
         ak[kt][ks] = frag_as<E>(f);
       }
     }
-    // V tile -> LDS, row-major with padded stride
-    __builtin_amdgcn_wave_barrier();
+  };
+  // V tile: global -> LDS, instruction i fills rows 8i..8i+7 (lane -> row 8i + lane/8, chunk position lane%8);
+  // position cp of row r holds source chunk cp ^ (4 * ((r >> 1) & 1)).
+  const int ldv_row = lane >> 3;
+  const int ldv_chunk = (lane & 7) ^ (((ldv_row >> 1) & 1) << 2);
+  const uint32_t voff = (uint32_t)ldv_row * (uint32_t)p.svn + ldv_chunk * 8;
+  auto load_v = [&](int64_t start) {
+    const bool partial = start + 64 > N;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      const int e = i * 64 + lane;
-      const int row = e >> 3, dch = e & 7;
-      uint4 raw = make_uint4(0, 0, 0, 0);
-      if (!partial || start + row < N) raw = *reinterpret_cast<const uint4*>(vp + (start + row) * p.svn + dch * 8);
-      *reinterpret_cast<uint4*>(vl + row * kVLd + dch * 8) = raw;
+      const E* vb = vp + (start + i * 8) * p.svn;  // wave-uniform
+      uint32_t off = voff;
+      if (partial) {
+        const int64_t last = N - 1 - start - i * 8;  // may be negative: whole group beyond N
+        const int64_t r = ldv_row < last ? ldv_row : last;
+        off = (uint32_t)(int32_t)(r * p.svn) + ldv_chunk * 8;
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + (int32_t)off),
+                                       (__attribute__((address_space(3))) void*)(vl + i * 512), 16, 0, 0);
     }
+  };
+  // per-lane byte offset of the transposed V read inside a 16-key group, for head_dim half dt = 0 (dt = 1: ^ 64)
+  const int i16 = lane & 15;
+  const int tr_row = 4 * hh + (i16 >> 2);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
+  const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
 
+  // One tile: S^T and softmax per query half; the next tile's K loads are issued into the same registers as soon
+  // as the second half's S^T MFMAs have consumed them; PV from the LDS tile; then the next tile's V load into the
+  // same LDS buffer.  `next` < 0: no further tile.
+  V8 ak[2][4];
+  auto tile = [&](int64_t start, int64_t next) {
+    const bool partial = start + 64 > N;
     V8 pf[2][2][2];  // P^T operands [qt][kt][jj]
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
-      f32x16 st[2];
+      f32x16 st[2];  // [kt]
 #pragma unroll
       for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
@@ -158,23 +211,33 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) st[kt] = MfmaT<E>::mma(ak[kt][ks], bq[qt][ks], st[kt]);
       }
-      if (partial) {
+      if (qt == 1 && next >= 0) load_k(ak, next);
+      if (partial) {  // keys at or beyond N: register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
+        const int lim = (int)(N - start) - 4 * hh;
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int64_t key = start + kt * 32 + hh * 4 + 8 * (r >> 2) + (r & 3);
-            if (key >= N) st[kt][r] = -INFINITY;
-          }
+          for (int r = 0; r < 16; r++)
+            if (kt * 32 + 8 * (r >> 2) + (r & 3) >= lim) st[kt][r] = -INFINITY;
       }
       float mx = st[0][0];
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
-      mx = xhalf_max(mx);
-      const float m_new = fmaxf(m_i[qt], mx * sl2);
-      const float alpha = __builtin_amdgcn_exp2f(m_i[qt] - m_new);
+      mx = xhalf_max(mx) * sl2;
+      const bool grow = mx > m_i[qt] + kRescaleSlack;  // true on the first tile (m_i = -inf)
+      if (__any(grow)) {
+        const float m_new = grow ? mx : m_i[qt];
+        const float alpha = __builtin_amdgcn_exp2f(m_i[qt] - m_new);  // 1 where the maximum stays
+        m_i[qt] = m_new;
+        l_i[qt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) ot[dt][qt][r] *= alpha;
+      }
+      const float m_use = m_i[qt];
       float rowsum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; kt++) {
@@ -183,43 +246,56 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
           V8 pk;
 #pragma unroll
           for (int e = 0; e < 8; e++) {
-            const float pv = __builtin_amdgcn_exp2f(fmaf(st[kt][8 * jj + e], sl2, -m_new));
+            const float pv = __builtin_amdgcn_exp2f(fmaf(st[kt][8 * jj + e], sl2, -m_use));
             rowsum += pv;
             pk[e] = (E)pv;
           }
           pf[qt][kt][jj] = pk;
         }
       }
-      l_i[qt] = l_i[qt] * alpha + rowsum;
-      m_i[qt] = m_new;
+      l_i[qt] += rowsum;
+    }
+
+    if (partial) {  // last, ragged key block: wait for the tile, then clear the rows beyond N
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      const int nvalid = (int)(N - start);
 #pragma unroll
-      for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) ot[dt][qt][r] *= alpha;
+      for (int i = 0; i < 8; i++)
+        if (i * 8 + ldv_row >= nvalid) *reinterpret_cast<uint4*>(vl + i * 512 + lane * 8) = make_uint4(0, 0, 0, 0);
     }
 
     // O^T += V^T P^T.  k-step (kt,jj) contracts keys kt*32 + 16jj + {4hh..4hh+3, 8+4hh..8+4hh+3}.
-    __builtin_amdgcn_wave_barrier();
+    const char* vbase = reinterpret_cast<const char*>(vl);
 #pragma unroll
     for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
       for (int jj = 0; jj < 2; jj++) {
 #pragma unroll
         for (int dt = 0; dt < 2; dt++) {
-          const E* a0 = vl + (kt * 32 + jj * 16 + tr_row) * kVLd + dt * 32 + tr_col;
+          const char* a0 = vbase + (tr_off ^ (dt * 64)) + (kt * 32 + jj * 16) * 128;
           Frag16B f;
           f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
-          f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * kVLd));
+          f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
           const V8 vf = frag_as<E>(f);
 #pragma unroll
           for (int qt = 0; qt < 2; qt++) ot[dt][qt] = MfmaT<E>::mma(vf, pf[qt][kt][jj], ot[dt][qt]);
         }
       }
     }
+    if (next >= 0) load_v(next);
+  };
+
+  int64_t start = next_start();
+  load_k(ak, start);
+  load_v(start);
+  while (remaining > 0) {
+    remaining--;
+    const int64_t next = remaining > 0 ? next_start() : -1;
+    tile(start, next);
+    start = next;
   }
 
   // epilogue
-  E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
     const float l = xhalf_sum(l_i[qt]);
