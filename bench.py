@@ -37,6 +37,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=1, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
+    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge"],
+                    help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
 
 
@@ -99,6 +101,25 @@ def main() -> int:
         out = s3r.gated_merge(o_cmp, o_sel, gd, block)
         mark(4)
         return out
+
+    if args.only:
+        with torch.no_grad():
+            qc, kc, vc = s3r.pool_mean(qd, block), s3r.pool_mean(kd, block), s3r.pool_mean(vd, block)
+            o_cmp, idx = s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat)
+            o_sel = s3r.select_attn(qd, kd, vd, idx, block)
+            stage = {
+                "pool": lambda: s3r.pool_mean(qd, block),
+                "compressed_topk": lambda: s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat),
+                "select": lambda: s3r.select_attn(qd, kd, vd, idx, block),
+                "merge": lambda: s3r.gated_merge(o_cmp, o_sel, gd, block),
+            }[args.only]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                stage()
+            torch.cuda.synchronize()
+            print(f"{args.only}: {(time.perf_counter() - t0) * 1e3 / args.steps:.4f} ms per launch", file=sys.stderr)
+        return 0
 
     with torch.no_grad():
         for _ in range(args.warmup):

@@ -110,7 +110,7 @@ def test_compressed_matches_oracle(dtype, lq, lk):
     o, idx, scores, lse = s3r.compressed_attn_topk(q.to(DEV), kk.to(DEV), v.to(DEV), k, return_scores=True, return_lse=True)
     o_ref, lse_ref, s_ref = oracle.compressed_attention(q, kk, v, out_dtype=torch.float32)
     assert max_abs(o, o_ref) <= TOL[dtype]
-    assert max_abs(lse, lse_ref) <= 1e-4
+    assert max_abs(lse, lse_ref) <= (1e-4 if dtype == torch.float32 else 2e-3)  # 16-bit: row sums are over rounded probabilities
     assert max_abs(scores, s_ref) <= 1e-4                           # same products, different summation order
     # indices are exact for the scores the kernel produced
     np.testing.assert_array_equal(idx.cpu().numpy(), oracle.topk_from_scores(scores.cpu(), k))
@@ -154,7 +154,7 @@ def test_select_matches_oracle(dtype, n, block, k):
     o_ref, lse_ref = oracle.select_attention(q, kk, v, idx, block, out_dtype=torch.float32, return_lse=True)
     assert o.dtype == dtype and o.shape == q.shape
     assert max_abs(o, o_ref) <= TOL[dtype]
-    assert max_abs(lse, lse_ref) <= 1e-4
+    assert max_abs(lse, lse_ref) <= (1e-4 if dtype == torch.float32 else 2e-3)  # 16-bit: row sums are over rounded probabilities
 
 
 def test_select_fixture(golden):
@@ -173,6 +173,34 @@ def test_select_empty_row_gives_zeros_and_strided_inputs_work():
     assert torch.count_nonzero(o[:, :, :64]) == 0
     o_ref = oracle.select_attention(q.cpu(), k.cpu(), v.cpu(), idx, 64, out_dtype=torch.float32)
     assert max_abs(o, o_ref) <= 2e-2
+
+
+@pytest.mark.parametrize("kernel", ["basic", "pipe"])
+def test_select_handles_scores_far_above_the_first_tile(kernel):
+    """The MFMA kernels take the first tile's row maximum as the softmax reference; when later tiles exceed it by
+    more than fp32 can hold they must fall back to the online softmax.  Block 0 listed first has tiny scores,
+    block 2 has logits around +140 in base-2 units above them (exp2 overflows fp32)."""
+    import subprocess, sys, textwrap
+    code = textwrap.dedent(f"""
+        import os, sys, torch
+        os.environ["S3R_SELECT_KERNEL"] = "{kernel}"
+        sys.path.insert(0, ".")
+        import oracle, speed3r_amd as s3r
+        g = torch.Generator().manual_seed(5)
+        n = 256
+        q = (torch.randn((1, 2, n, 64), generator=g)).to(torch.bfloat16)
+        k = (torch.randn((1, 2, n, 64), generator=g) * 0.01).to(torch.bfloat16)
+        k[:, :, 128:192] = (q[:, :, 0:64] * 12.0)          # block 2: logits ~140 (base 2) above block 0's
+        v = torch.randn((1, 2, n, 64), generator=g).to(torch.bfloat16)
+        idx = torch.tensor([[0, 2, 1], [1, 0, 3], [2, 3, 0], [3, 1, 2]], dtype=torch.int32).view(1, 1, 4, 3).expand(1, 2, 4, 3).contiguous()
+        o = s3r.select_attn(q.cuda(), k.cuda(), v.cuda(), idx.cuda(), 64)
+        ref = oracle.select_attention(q, k, v, idx, 64, out_dtype=torch.float32)
+        err = (o.float().cpu() - ref).abs().max().item()
+        assert torch.isfinite(o.float()).all() and err <= 2e-2, err
+        print("ok", err)
+    """)
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
 
 
 def test_forward_only_guard():
