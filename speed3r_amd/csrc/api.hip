@@ -26,7 +26,7 @@ extern "C" const char* s3r_version(void) { return "speed3r_hip 0.1 gfx950"; }
 
 extern "C" const char* s3r_last_error(void) { return last_error_buffer(); }
 
-extern "C" int s3r_capabilities(void) { return 0; }
+extern "C" int s3r_capabilities(void) { return S3R_CAP_FUSED_TOPK; }
 
 extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void* v, void* o, float* lse, int32_t* topk_idx,
                                         float* scores, int B, int H, int Lq, int Lk, int D, int K,

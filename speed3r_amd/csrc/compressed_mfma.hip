@@ -1,38 +1,59 @@
 // Compressed-branch attention on the gfx950 matrix cores (bf16 / fp16 I/O, head_dim 64):
-// dense non-causal flash attention over the pooled tokens, with the raw score tile
-// optionally written out for the block selection.
+// dense non-causal flash attention over the pooled tokens, plus the exact top-k block
+// selection, either fused into the same pass or from a score matrix written to HBM.
 //
-// A 256-thread workgroup owns 128 query rows of one head, 32 per wavefront, and walks all
-// key tiles of 64 pooled tokens.  K and V tiles are staged once per workgroup in LDS
-// (global -> registers one tile ahead -> LDS) and shared by the four waves.  Per wave and
-// tile: S^T = K Q^T with v_mfma_f32_32x32x16 (one query per lane, see select_mfma.hip for
-// the layout argument), base-2 online softmax in fp32, P rounded to the I/O dtype,
-// O^T += V^T P^T with V^T fragments read through ds_read_b64_tr_b16.
+// A 256-thread workgroup owns 128 query rows of one head, 32 per wavefront, and walks all key
+// tiles of 64 pooled tokens.  K and V tiles are staged once per workgroup in LDS (global ->
+// registers two tiles ahead -> LDS one tile ahead, two LDS buffers, one barrier per tile) and
+// shared by the four waves.  Rows are 128 bytes without padding; 16-byte chunks are stored
+// XOR-swizzled (K: chunk ^ (row & 7) for the 16-byte operand reads, V: halves swapped on rows
+// 2,3 mod 4 for the transposed reads) so that LDS reads are bank-conflict free.
+// Per wave and tile: S^T = K Q^T with v_mfma_f32_32x32x16 (one query per lane and its partner
+// lane ^ 32, 32 of the tile's 64 keys in each lane's registers), base-2 online softmax in
+// fp32, P rounded to the I/O dtype, O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16.
+//
+// Fused selection.  Every lane keeps the exact top-K of the keys IT sees (half of each tile):
+// a descending sorted list of K 64-bit keys, key = sortable(bits(score)) << 32 | (Lk-1-col),
+// in registers.  Scores are first filtered against the score of the list's last entry (one
+// compare per score; survivors are appended to a small per-lane queue in LDS).  When some
+// lane's queue is more than half full, all lanes merge their queues into their lists with a
+// register-resident bitonic network (no divergence: every lane runs the same network on its
+// own data) and refresh their thresholds.  At the end the two lanes of a query merge their
+// lists and lane < 32 writes the K indices in descending key order.  The filter is
+// conservative (anything that could enter passes), the network compares full 64-bit keys,
+// so the result is the same unique top-K as a sort of the whole row.
 #include "s3r_common.h"
 #include "attn_params.h"
+#include <type_traits>
+#include <utility>
 
 namespace s3r {
+namespace cmp {
 
-template <typename E> struct MfmaC;
-template <> struct MfmaC<bf16_t> {
+template <typename E> struct Mma;
+template <> struct Mma<bf16_t> {
   typedef bf16x8 V8;
   static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 };
-template <> struct MfmaC<f16_t> {
+template <> struct Mma<f16_t> {
   typedef f16x8 V8;
   static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
 };
 
-union FragC {
+union Frag {
   uint4 u;
   bf16x8 b;
   f16x8 h;
   s16x4 s[2];
 };
-template <typename E> __device__ __forceinline__ typename MfmaC<E>::V8 fragc_as(const FragC& f);
-template <> __device__ __forceinline__ bf16x8 fragc_as<bf16_t>(const FragC& f) { return f.b; }
-template <> __device__ __forceinline__ f16x8 fragc_as<f16_t>(const FragC& f) { return f.h; }
+template <typename E> __device__ __forceinline__ typename Mma<E>::V8 as_v8(const Frag& f);
+template <> __device__ __forceinline__ bf16x8 as_v8<bf16_t>(const Frag& f) { return f.b; }
+template <> __device__ __forceinline__ f16x8 as_v8<f16_t>(const Frag& f) { return f.h; }
 
+__device__ __forceinline__ uint32_t xh_swap(uint32_t x) {  // value held by lane ^ 32
+  auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  return (threadIdx.x & 32) ? r[0] : r[1];
+}
 __device__ __forceinline__ float xh_max(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
@@ -42,13 +63,57 @@ __device__ __forceinline__ float xh_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-constexpr int kCLd = 72;  // LDS row stride in elements (144 bytes)
+// ---- register-resident bitonic networks on 64-bit keys (descending order) ----
+__device__ __forceinline__ void cex_desc(uint64_t& a, uint64_t& b) {  // a = max, b = min
+  const bool gt = a > b;
+  const uint64_t hi = gt ? a : b;
+  const uint64_t lo = gt ? b : a;
+  a = hi;
+  b = lo;
+}
+template <int N> __device__ __forceinline__ void bitonic_merge_desc(uint64_t (&x)[N]) {  // x bitonic -> descending
+#pragma unroll
+  for (int d = N / 2; d >= 1; d >>= 1)
+#pragma unroll
+    for (int i = 0; i < N; i++)
+      if ((i & d) == 0) cex_desc(x[i], x[i | d]);
+}
+template <int N> __device__ __forceinline__ void bitonic_sort_desc(uint64_t (&x)[N]) {
+#pragma unroll
+  for (int k = 2; k <= N; k <<= 1)
+#pragma unroll
+    for (int d = k / 2; d >= 1; d >>= 1)
+#pragma unroll
+      for (int i = 0; i < N; i++) {
+        const int j = i ^ d;
+        if (j > i) {
+          if ((i & k) == 0 || k == N) {  // descending run (the last stage sorts everything descending)
+            cex_desc(x[i], x[j]);
+          } else {  // ascending run
+            cex_desc(x[j], x[i]);
+          }
+        }
+      }
+}
+// top-N of (descending a) U (descending b) -> a, descending
+template <int N> __device__ __forceinline__ void merge_top_desc(uint64_t (&a)[N], const uint64_t (&b)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; i++) a[i] = a[i] > b[N - 1 - i] ? a[i] : b[N - 1 - i];  // half-cleaner: a is now bitonic
+  bitonic_merge_desc<N>(a);
+}
 
-template <typename E>
-__global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
-  typedef typename MfmaC<E>::V8 V8;
-  __shared__ __attribute__((aligned(16))) E Ks[64 * kCLd];
-  __shared__ __attribute__((aligned(16))) E Vs[64 * kCLd];
+constexpr int kTile = 64 * 64;  // elements per LDS tile
+constexpr int kQSlots = 16;     // LDS queue slots per lane: kQSlots-1 entries and one dump slot for non-survivors
+constexpr int kQCap = kQSlots;  // width of the merge network (entry kQSlots-1 is always empty)
+
+template <typename E, int KTOP /* 0: no fused selection */>
+__global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
+  typedef typename Mma<E>::V8 V8;
+  constexpr bool FUSED = KTOP > 0;
+  constexpr int KL = FUSED ? KTOP : 1;  // list length per lane
+  __shared__ __attribute__((aligned(1024))) E Ks[2][kTile];
+  __shared__ __attribute__((aligned(1024))) E Vs[2][kTile];
+  __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][FUSED ? kQSlots : 1][64];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -69,10 +134,10 @@ __global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
   V8 bq[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ks++) {
-    FragC f;
+    Frag f;
     f.u = make_uint4(0, 0, 0, 0);
     if (qvalid) f.u = *reinterpret_cast<const uint4*>(qp + qrow * p.sqm + ks * 16 + hh * 8);
-    bq[ks] = fragc_as<E>(f);
+    bq[ks] = as_v8<E>(f);
   }
 
   f32x16 ot[2];
@@ -83,49 +148,96 @@ __global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
   float m_i = -INFINITY, l_i = 0.f;
   const float sl2 = p.scale * 1.4426950408889634f;
 
-  const int tr_row = 4 * hh + ((lane & 15) >> 2);
-  const int tr_col = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-
-  // cooperative tile staging: thread owns 16-byte chunks e = tid and tid + 256 of each 64x64 tile
-  const int ld_row0 = tid >> 3, ld_dch = tid & 7;  // second chunk: row + 32
+  // ---- tile staging: thread owns chunk rows ld_row, ld_row+32 at chunk position ld_pos of both tiles ----
+  const int ld_row = tid >> 3, ld_pos = tid & 7;
   uint4 kr[2], vr[2];
-  auto prefetch = [&](int64_t start) {
+  auto fetch = [&](int64_t start) {  // global -> registers; rows beyond Lk re-read the last row (they are masked)
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      const int64_t row = start + ld_row0 + 32 * i;
-      kr[i] = make_uint4(0, 0, 0, 0);
-      vr[i] = make_uint4(0, 0, 0, 0);
-      if (row < Lk) {
-        kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ld_dch * 8);
-        vr[i] = *reinterpret_cast<const uint4*>(vp + row * p.svn + ld_dch * 8);
-      }
+      const int r = ld_row + 32 * i;
+      int64_t row = start + r;
+      row = row < Lk ? row : Lk - 1;
+      kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
+      vr[i] = *reinterpret_cast<const uint4*>(vp + row * p.svn + ((ld_pos ^ (((r >> 1) & 1) << 2)) * 8));
     }
+  };
+  auto stash = [&](int buf) {  // registers -> LDS
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int r = ld_row + 32 * i;
+      *reinterpret_cast<uint4*>(&Ks[buf][r * 64 + ld_pos * 8]) = kr[i];
+      *reinterpret_cast<uint4*>(&Vs[buf][r * 64 + ld_pos * 8]) = vr[i];
+    }
+  };
+  // per-lane LDS read offsets (bytes)
+  const int i16 = lane & 15;
+  const int tr_row = 4 * hh + (i16 >> 2);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
+  const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
+
+  // ---- fused selection state ----
+  uint64_t list[KL];  // descending
+#pragma unroll
+  for (int i = 0; i < KL; i++) list[i] = 0;
+  float thr = __uint_as_float(0xFFFFFFFFu);  // a NaN: "s < thr" is false for every s, so everything passes
+  int qn = 0;
+  uint2* qlane = FUSED ? &queue[wave][0][lane] : nullptr;  // entry e at qlane[e * 64]
+  const uint32_t lkm1 = (uint32_t)(Lk - 1);
+
+  auto drain = [&]() {  // merge this lane's queue into its list; every lane runs the same network
+    uint64_t cand[kQCap];
+#pragma unroll
+    for (int e = 0; e < kQCap; e++) {
+      const uint2 v = qlane[e * 64];
+      const uint64_t key = ((uint64_t)sortable_key(__uint_as_float(v.x)) << 32) | (uint64_t)(lkm1 - v.y);
+      cand[e] = e < qn ? key : 0;
+    }
+    bitonic_sort_desc<kQCap>(cand);
+    if constexpr (KL == kQCap) {
+      merge_top_desc<KL>(list, cand);
+    } else if constexpr (KL < kQCap) {  // keep the KL best of list U cand: widen the list, merge, truncate
+      uint64_t wide[kQCap];
+#pragma unroll
+      for (int i = 0; i < kQCap; i++) wide[i] = i < KL ? list[i] : 0;
+      merge_top_desc<kQCap>(wide, cand);
+#pragma unroll
+      for (int i = 0; i < KL; i++) list[i] = wide[i];
+    } else {  // KL > kQCap: merge the candidates into the two (or more) halves' worth of list
+      uint64_t wide[KL];
+#pragma unroll
+      for (int i = 0; i < KL; i++) wide[i] = i < kQCap ? cand[i] : 0;
+      merge_top_desc<KL>(list, wide);
+    }
+    qn = 0;
+    // threshold = score of the list's last entry (key 0, a filler, maps to a NaN: everything passes)
+    const uint32_t k32 = (uint32_t)(list[KL - 1] >> 32);
+    thr = __uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu));
   };
 
   const int ntiles = (int)((Lk + 63) / 64);
-  prefetch(0);
+  fetch(0);
+  stash(0);
+  if (ntiles > 1) fetch(64);
+
   for (int t = 0; t < ntiles; t++) {
+    const int buf = t & 1;
     const int64_t start = (int64_t)t * 64;
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      *reinterpret_cast<uint4*>(Ks + (ld_row0 + 32 * i) * kCLd + ld_dch * 8) = kr[i];
-      *reinterpret_cast<uint4*>(Vs + (ld_row0 + 32 * i) * kCLd + ld_dch * 8) = vr[i];
-    }
-    __syncthreads();
-    if (t + 1 < ntiles) prefetch(start + 64);
+    __syncthreads();  // tile t visible in LDS; everyone is done with buffer buf^1
+    if (t + 1 < ntiles) stash(buf ^ 1);
+    if (t + 2 < ntiles) fetch(start + 128);
     const bool partial = start + 64 > Lk;
 
     f32x16 st[2];
+    const char* kbase = reinterpret_cast<const char*>(&Ks[buf][0]);
 #pragma unroll
     for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
-        FragC f;
-        f.u = *reinterpret_cast<const uint4*>(Ks + (kt * 32 + c) * kCLd + ks * 16 + hh * 8);
-        st[kt] = MfmaC<E>::mma(fragc_as<E>(f), bq[ks], st[kt]);
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
+        st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
       }
     }
 
@@ -147,14 +259,35 @@ __global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
         }
     }
 
+    const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
+    if constexpr (FUSED) {
+      // filter the raw scores against the lane's threshold; survivors go to the lane's queue
+      const uint32_t col0 = (uint32_t)start + 4 * hh;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
+#pragma unroll
+        for (int e8 = 0; e8 < 8; e8++) {
+          const int kt = g >> 1, r = (g & 1) * 8 + e8;
+          const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
+          const float s = st[kt][r];
+          bool pass = !(s < thr);
+          if (partial) pass = pass && (koff < lim);
+          if (__any(pass)) {
+            uint2* dst = pass ? qlane + qn * 64 : qlane + (kQSlots - 1) * 64;  // non-survivors write the dump slot
+            *dst = make_uint2(__float_as_uint(s), col0 + koff);
+            qn += pass ? 1 : 0;
+          }
+        }
+        if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
+      }
+    }
+
     if (partial) {
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int64_t key = start + kt * 32 + hh * 4 + 8 * (r >> 2) + (r & 3);
-          if (key >= Lk) st[kt][r] = -INFINITY;
-        }
+        for (int r = 0; r < 16; r++)
+          if (kt * 32 + 8 * (r >> 2) + (r & 3) >= lim) st[kt][r] = -INFINITY;
     }
     float mx = st[0][0];
 #pragma unroll
@@ -186,17 +319,18 @@ __global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
 
+    const char* vbase = reinterpret_cast<const char*>(&Vs[buf][0]);
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
         for (int dt = 0; dt < 2; dt++) {
-          const E* a0 = Vs + (kt * 32 + jj * 16 + tr_row) * kCLd + dt * 32 + tr_col;
-          FragC f;
+          const char* a0 = vbase + (tr_off ^ (dt * 64)) + (kt * 32 + jj * 16) * 128;
+          Frag f;
           f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
-          f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * kCLd));
-          ot[dt] = MfmaC<E>::mma(fragc_as<E>(f), pf[kt][jj], ot[dt]);
+          f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+          ot[dt] = Mma<E>::mma(as_v8<E>(f), pf[kt][jj], ot[dt]);
         }
   }
 
@@ -216,22 +350,61 @@ __global__ __launch_bounds__(256) void compressed_mfma_kernel(AttnParams p) {
     if (p.lse != nullptr && hh == 0)
       p.lse[((int64_t)b * p.H + h) * Lq + qrow] = l > 0.f ? (m_i + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
   }
+
+  if constexpr (FUSED) {
+    drain();
+    // the partner lane's list, then the K best of both, descending
+    uint64_t other[KL];
+#pragma unroll
+    for (int i = 0; i < KL; i++) {
+      const uint32_t lo = xh_swap((uint32_t)list[i]);
+      const uint32_t hi = xh_swap((uint32_t)(list[i] >> 32));
+      other[i] = ((uint64_t)hi << 32) | lo;
+    }
+    merge_top_desc<KL>(list, other);
+    if (qvalid && hh == 0) {
+      int32_t* irow = p.topk_idx + (((int64_t)b * p.H + h) * Lq + qrow) * KL;
+#pragma unroll
+      for (int i = 0; i < KL; i++) irow[i] = (int32_t)(lkm1 - (uint32_t)list[i]);
+    }
+  }
 }
 
-int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream) {
-  if (p.topk_idx != nullptr && p.scores == nullptr)
-    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection not built; pass a scores buffer");
+template <typename E>
+static int launch_e(const AttnParams& p, bool fused, hipStream_t st) {
   const int64_t nqg = (p.Lq + 127) / 128;
   if (nqg > 0x7fffffffLL || (int64_t)p.B * p.H > 65535) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: grid too large");
-  hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)nqg, (unsigned)(p.B * p.H)), blk(256);
-  if (dtype == S3R_BF16)
-    hipLaunchKernelGGL(compressed_mfma_kernel<bf16_t>, grid, blk, 0, st, p);
-  else
-    hipLaunchKernelGGL(compressed_mfma_kernel<f16_t>, grid, blk, 0, st, p);
-  int rc = check_launch("compressed_mfma_kernel");
+  if (!fused) {
+    hipLaunchKernelGGL((compressed_mfma_kernel<E, 0>), grid, blk, 0, st, p);
+  } else {
+    switch (p.K) {
+      case 1: hipLaunchKernelGGL((compressed_mfma_kernel<E, 1>), grid, blk, 0, st, p); break;
+      case 2: hipLaunchKernelGGL((compressed_mfma_kernel<E, 2>), grid, blk, 0, st, p); break;
+      case 4: hipLaunchKernelGGL((compressed_mfma_kernel<E, 4>), grid, blk, 0, st, p); break;
+      case 8: hipLaunchKernelGGL((compressed_mfma_kernel<E, 8>), grid, blk, 0, st, p); break;
+      case 16: hipLaunchKernelGGL((compressed_mfma_kernel<E, 16>), grid, blk, 0, st, p); break;
+      case 32: hipLaunchKernelGGL((compressed_mfma_kernel<E, 32>), grid, blk, 0, st, p); break;
+      default: return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}");
+    }
+  }
+  return check_launch("compressed_mfma_kernel");
+}
+
+}  // namespace cmp
+
+bool compressed_fused_topk_available(int K) { return K == 1 || K == 2 || K == 4 || K == 8 || K == 16 || K == 32; }
+
+int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  // fused selection when indices are wanted and no score buffer is given; with a score buffer the indices come
+  // from exactly the stored values through the row-wise kernel
+  const bool fused = p.topk_idx != nullptr && p.scores == nullptr;
+  if (fused && !compressed_fused_topk_available(p.K))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}; pass a scores buffer");
+  int rc = dtype == S3R_BF16 ? cmp::launch_e<bf16_t>(p, fused, st) : cmp::launch_e<f16_t>(p, fused, st);
   if (rc != S3R_OK) return rc;
-  if (p.topk_idx != nullptr)
+  if (p.topk_idx != nullptr && !fused)
     rc = s3r_topk_rows(p.scores, p.topk_idx, (int64_t)p.B * p.H * p.Lq, (int)p.Lk, p.Lk, p.K, stream);
   return rc;
 }

@@ -123,6 +123,41 @@ def test_compressed_fixture(golden):
     assert max_abs(scores, torch.from_numpy(golden["cmp_scores"])) <= 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("k", [1, 2, 4, 8, 16, 32])
+@pytest.mark.parametrize("lq,lk", [(150, 150), (64, 64), (5, 5), (100, 300), (300, 100), (1041, 1041), (130, 4164)])
+def test_fused_selection_equals_selection_from_stored_scores(dtype, k, lq, lk):
+    """The fused top-k never sees HBM scores; the same kernel with a score buffer produces bit-identical
+    scores, so both index sets must agree bit for bit with the oracle's order on those scores."""
+    h = 2
+    q = _randn((1, h, lq, 64), lq + k, dtype, 0.5).to(DEV)
+    kk = _randn((1, h, lk, 64), lk + 1, dtype, 0.5)
+    kk[:, :, lk // 2:] = kk[:, :, :lk - lk // 2]          # duplicated keys: exact score ties, lowest column must win
+    kk = kk.to(DEV)
+    v = _randn((1, h, lk, 64), lk + 2, dtype).to(DEV)
+    o_f, idx_f = s3r.compressed_attn_topk(q, kk, v, k, materialize_scores=False)
+    o_m, idx_m, scores = s3r.compressed_attn_topk(q, kk, v, k, return_scores=True)
+    want = oracle.topk_from_scores(scores.cpu(), k)
+    np.testing.assert_array_equal(idx_m.cpu().numpy(), want)
+    np.testing.assert_array_equal(idx_f.cpu().numpy(), want)
+    assert torch.equal(o_f, o_m)
+
+
+def test_fused_selection_special_scores():
+    """Zero queries give all-zero scores (every column ties: indices 0..K-1); a huge key gives +inf scores."""
+    lk = 200
+    q = torch.zeros((1, 1, 70, 64), dtype=torch.bfloat16, device=DEV)
+    kk = _randn((1, 1, lk, 64), 3, torch.bfloat16).to(DEV)
+    v = _randn((1, 1, lk, 64), 4, torch.bfloat16).to(DEV)
+    _, idx = s3r.compressed_attn_topk(q, kk, v, 16, materialize_scores=False)
+    assert torch.equal(idx.cpu(), torch.arange(16, dtype=torch.int32).expand(1, 1, 70, 16))
+    q = _randn((1, 1, 70, 64), 5, torch.bfloat16).to(DEV)
+    kk[0, 0, 150] = 3e38
+    _, idx_f = s3r.compressed_attn_topk(q, kk, v, 8, materialize_scores=False)
+    _, idx_m, scores = s3r.compressed_attn_topk(q, kk, v, 8, return_scores=True)
+    np.testing.assert_array_equal(idx_f.cpu().numpy(), oracle.topk_from_scores(scores.cpu(), 8))
+
+
 def test_flash_attn_topk_func_signature():
     q = _randn((1, 2, 200, 64), 5, torch.bfloat16, 0.5)
     o, idx = s3r.flash_attn_topk_func(q.to(DEV), q.to(DEV), q.to(DEV), 16)
