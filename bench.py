@@ -35,7 +35,7 @@ def parse_args():
     ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--topk", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-heads", type=int, default=1, help="heads of the workload the CPU baseline runs")
+    ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
     ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
@@ -135,12 +135,12 @@ def main() -> int:
         peak_mem = torch.cuda.max_memory_allocated()
 
     ms_per_step = wall * 1e3 / args.steps
+    nc = -(-n // block)
     kern_ms = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
     f_sel = workloads.selection_flops(n, topk)
     f_cmp = workloads.compressed_flops(n)
     sel_tflops = f_sel / (kern_ms["select"] * 1e-3) / 1e12
     es = 2 if cfg.dtype != torch.float32 else 4
-    nc = -(-n // block)
     pool_bytes = 3 * (n + nc) * 16 * 64 * es
     merge_bytes = (2 * n * 16 * 64 + n * 16 * 2 + nc * 16 * 64) * es
 
@@ -161,7 +161,8 @@ def main() -> int:
             "workload": f"{cfg.name}: {cfg.frames} frames x {workloads.TOKENS_PER_FRAME} tokens = {n} tokens, "
                         f"16 heads x 64, block {block}, top-k {topk}, B=1",
             "tokens": n, "heads": 16, "head_dim": 64, "block": block, "topk": topk,
-            "scores": "materialized" if (args.materialize_scores or not s3r._lib.lib_has_fused_topk()) else "fused",
+            "scores": "materialized" if (args.materialize_scores or 16 * nc * nc * 4 <= s3r.sparse_attn.ops.SCORE_BUFFER_LIMIT)
+                      else "fused",
         },
         "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
         "kernels_ms": kern_ms,

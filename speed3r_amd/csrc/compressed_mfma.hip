@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(1024))) E Ks[2][kTile];
   __shared__ __attribute__((aligned(1024))) E Vs[2][kTile];
   __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][FUSED ? kQSlots : 1][64];
+  __shared__ __attribute__((aligned(16))) float sstage[FUSED ? 1 : 4][FUSED ? 4 : 32 * 64];  // score-store staging (unfused launches)
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -241,22 +242,37 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
       }
     }
 
-    if (p.scores != nullptr && qvalid) {
-      float* srow = p.scores + (((int64_t)b * p.H + h) * Lq + qrow) * Lk + start;
+    if (p.scores != nullptr) {
+      float* sbase = p.scores + (((int64_t)b * p.H + h) * Lq + q0) * Lk + start;  // row 0 of this wave, column 0 of the tile
       const bool vec = ((Lk & 3) == 0) && !partial && ((reinterpret_cast<uintptr_t>(p.scores) & 15u) == 0);
+      if (vec) {
+        // transpose the 32 x 64 score tile through a wave-private LDS stage so that every store instruction
+        // writes four full 256-byte row segments (16-byte chunk ch of row r sits at chunk ch ^ (r & 15))
+        float* stg = &sstage[wave][0];
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++)
+        for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-          const int col = kt * 32 + 4 * hh + 8 * g4;
-          if (vec) {
-            *reinterpret_cast<float4*>(srow + col) = make_float4(st[kt][4 * g4], st[kt][4 * g4 + 1], st[kt][4 * g4 + 2], st[kt][4 * g4 + 3]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              if (start + col + e < Lk) srow[col + e] = st[kt][4 * g4 + e];
+          for (int g4 = 0; g4 < 4; g4++) {
+            const int ch = kt * 8 + 2 * g4 + hh;
+            *reinterpret_cast<float4*>(stg + c * 64 + ((ch ^ (c & 15)) * 4)) =
+                make_float4(st[kt][4 * g4], st[kt][4 * g4 + 1], st[kt][4 * g4 + 2], st[kt][4 * g4 + 3]);
           }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const int r = i * 4 + (lane >> 4), ch = lane & 15;
+          const float4 v4 = *reinterpret_cast<const float4*>(stg + r * 64 + ((ch ^ (r & 15)) * 4));
+          if (q0 + r < Lq) *reinterpret_cast<float4*>(sbase + (int64_t)r * Lk + ch * 4) = v4;
         }
+      } else if (qvalid) {
+        float* srow = sbase + (int64_t)c * Lk;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int col = kt * 32 + 4 * hh + 8 * (r >> 2) + (r & 3);
+            if (start + col < Lk) srow[col] = st[kt][r];
+          }
+      }
     }
 
     const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4

@@ -32,12 +32,22 @@ __global__ __launch_bounds__(256) void pool_mean_kernel(
   float acc[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; i++) acc[i] = 0.f;
-#pragma unroll 8
-  for (int r = r0; r < nvalid; r += rpw) {
-    uint4 raw = *reinterpret_cast<const uint4*>(base + (int64_t)r * sxn);
-    const T* e = reinterpret_cast<const T*>(&raw);
+  // batches of 8 loads issued back to back (rows beyond the block re-read its last row and are not added),
+  // so that 8 KB per wave are in flight instead of one load at a time
+  for (int r = r0; r < nvalid; r += 8 * rpw) {
+    uint4 raw[8];
 #pragma unroll
-    for (int i = 0; i < VEC; i++) acc[i] += to_f32(e[i]);
+    for (int u = 0; u < 8; u++) {
+      const int rr = r + u * rpw;
+      raw[u] = *reinterpret_cast<const uint4*>(base + (int64_t)(rr < nvalid ? rr : nvalid - 1) * sxn);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const T* e = reinterpret_cast<const T*>(&raw[u]);
+      const bool keep = r + u * rpw < nvalid;
+#pragma unroll
+      for (int i = 0; i < VEC; i++) acc[i] += keep ? to_f32(e[i]) : 0.f;
+    }
   }
   for (int off = lpr; off < 64; off <<= 1) {
 #pragma unroll
