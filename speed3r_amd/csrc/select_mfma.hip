@@ -91,14 +91,15 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
 
-constexpr int kVTile = 64 * 64;  // elements per LDS V buffer
-constexpr int kVBufs = 2;        // LDS V buffers per wave
+constexpr int kTile = 64 * 64;  // elements per LDS tile buffer (one K and one V buffer per wave)
 
 template <typename E>
 __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[4 * kVBufs * kVTile * 2];
+  // two separate arrays: the compiler then tells the K and V transfers apart when it counts outstanding loads
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k[4 * kTile * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v[4 * kTile * 2];
 
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -123,7 +124,8 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
   const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
   E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
   const int32_t* idx_row = p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
-  E* vl = reinterpret_cast<E*>(lds_raw) + wave * (kVBufs * kVTile);
+  E* kl = reinterpret_cast<E*>(lds_k) + wave * kTile;
+  E* vl = reinterpret_cast<E*>(lds_v) + wave * kTile;
 
   // index list: full tiles go through the pipeline, occurrences of the ragged last block come after it
   const int32_t my_idx = lane < p.K ? idx_row[lane] : -1;
@@ -192,25 +194,46 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
         dst[kt][ks] = as_v8<E>(f);
       }
   };
+  // K tile global -> LDS: LDS chunk (row, c') holds head_dim chunk c' ^ (row & 7); a lane quad stays inside one 64-byte
+  // half row on the global side, and the A-operand reads below (32 rows x one chunk) spread over all banks
   const int ldv_row = lane >> 3;
-  const int ldv_chunk = (lane & 7) ^ (((ldv_row >> 1) & 1) << 2);
-  const uint32_t voff = (uint32_t)ldv_row * (uint32_t)p.svn + ldv_chunk * 8;
-  auto load_v = [&](int buf, int64_t start) {
-    E* dst = vl + buf * kVTile;
+  // (buffer loads rather than global loads: the compiler then counts the outstanding transfers per LDS array)
+  const uint32_t klds_off = ((uint32_t)ldv_row * (uint32_t)p.skn + (((lane & 7) ^ (ldv_row & 7)) * 8)) * (uint32_t)sizeof(E);
+  const uint32_t k_step = 8u * (uint32_t)p.skn * (uint32_t)sizeof(E);  // 8 rows per transfer instruction
+  auto load_k_lds = [&](int64_t start) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const E* vb = vp + (start + i * 8) * p.svn;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + voff),
-                                       (__attribute__((address_space(3))) void*)(dst + i * 512), 16, 0, 0);
-    }
+    for (int i = 0; i < 8; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(kl + i * 512), 16, klds_off, i * k_step, 0, 0);
+  };
+  const int kr_off = c * 128 + ((hh ^ (c & 7)) << 4);
+  auto read_k = [&](V8 (&dst)[2][4]) {
+    const char* kbase = reinterpret_cast<const char*>(kl);
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(kbase + kt * 4096 + (kr_off ^ (ks << 5)));
+        dst[kt][ks] = as_v8<E>(f);
+      }
+  };
+  const int ldv_chunk = (lane & 7) ^ (((ldv_row >> 1) & 1) << 2);
+  const uint32_t voff = ((uint32_t)ldv_row * (uint32_t)p.svn + ldv_chunk * 8) * (uint32_t)sizeof(E);
+  const uint32_t v_step = 8u * (uint32_t)p.svn * (uint32_t)sizeof(E);
+  auto load_v = [&](int64_t start) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + start * p.svn), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(vl + i * 512), 16, voff, i * v_step, 0, 0);
   };
   const int i16 = lane & 15;
   const int tr_row = 4 * hh + (i16 >> 2);
   const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
   const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
   // all V^T fragments of one tile: [kt][jj][dt], k-step (kt,jj) = keys kt*32 + 16jj + {4hh.., 8+4hh..}
-  auto read_v = [&](V8 (&vfr)[2][2][2], int buf) {
-    const char* vbase = reinterpret_cast<const char*>(vl + buf * kVTile);
+  auto read_v = [&](V8 (&vfr)[2][2][2]) {
+    const char* vbase = reinterpret_cast<const char*>(vl);
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -234,9 +257,9 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
   };
 
   // PV of a finished probability tile without anything to overlap it with
-  auto pv_only = [&](const V8 (&pp)[2][2][2], int buf) {
+  auto pv_only = [&](const V8 (&pp)[2][2][2]) {
     V8 vfr[2][2][2];
-    read_v(vfr, buf);
+    read_v(vfr);
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -257,11 +280,12 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
         for (int ks = 0; ks < 4; ks++) s[qt][kt] = Mma<E>::mma(kk[kt][ks], bq[qt][ks], s[qt][kt]);
       }
   };
-  // One tile of the fast loop: S^T and exponentials per query half; as soon as the second half's S^T MFMAs
-  // have consumed the K registers the next tile's K loads (same registers) and V load (other LDS buffer) are
-  // issued; then PV for both halves from this tile's LDS buffer.
-  auto fast_tile = [&](int buf, int64_t next) {
+  // One tile of the fast loop: K from LDS into registers, S^T and exponentials per query half, PV from the V buffer.
+  // The transfer of the next K tile starts once the first S^T MFMAs have consumed this tile's K registers (the K
+  // buffer is free from then on) and that of the next V tile after the PV reads: each has about one tile of time.
+  auto fast_tile = [&](int64_t next) {
     const float mneg[2] = {-m_i[0], -m_i[1]};
+    read_k(ak[0]);
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
 #pragma unroll
@@ -271,9 +295,10 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) st[0][qt][kt] = Mma<E>::mma(ak[0][kt][ks], bq[qt][ks], st[0][qt][kt]);
       }
-      if (qt == 1) {
-        load_k(ak[0], next);
-        load_v(buf ^ 1, next);
+      if (qt == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_k_lds(next);
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
@@ -289,7 +314,9 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
             l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
           }
     }
-    pv_only(pf[0], buf);
+    __builtin_amdgcn_sched_barrier(0);
+    pv_only(pf[0]);
+    load_v(next);
   };
   // Unpipelined stage with a true online softmax: one key tile (possibly ragged) from global memory.
   auto robust_tile = [&](int64_t start) {
@@ -307,7 +334,7 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
         ak[0][kt][ks] = as_v8<E>(f);
       }
     }
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): earlier reads of LDS buffer 0 are done
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): earlier reads of the V buffer are done
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const int row = i * 8 + ldv_row;
@@ -347,7 +374,7 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
             l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
           }
     }
-    pv_only(pf[0], 0);
+    pv_only(pf[0]);
   };
   auto reset_state = [&]() {
 #pragma unroll
@@ -364,8 +391,8 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
   if (n_full > 0) {
     // first tile: its row maxima become the softmax reference
     const int64_t s0 = pop_start();
-    load_k(ak[0], s0);
-    load_v(0, s0);
+    load_k_lds(s0);
+    load_v(s0);
     int64_t last_start = s0;
     auto pop_or_last = [&]() -> int64_t {  // branch-free: next full tile, or the last one again
       const bool any = todo != 0;
@@ -375,14 +402,12 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
       last_start = any ? s : last_start;
       return last_start;
     };
+    read_k(ak[0]);
     scores_only(st[0], ak[0]);
     m_i[0] = row_max(st[0][0]);
     m_i[1] = row_max(st[0][1]);
-    int buf = 0;
-    for (int i = n_full; i > 0; i--) {  // past the end of the list the prefetch re-reads the last tile
-      fast_tile(buf, pop_or_last());
-      buf ^= 1;
-    }
+    for (int i = n_full; i > 0; i--)  // past the end of the list the prefetch re-reads the last tile
+      fast_tile(pop_or_last());
     // a reference that was too low shows up as a huge or non-finite row sum
     const float big = 1.2676506e30f;  // 2^100
     redo = __any(!(l_i[0] < big) || !(l_i[1] < big));

@@ -41,6 +41,12 @@ template <> struct Mma<bf16_t> {
   typedef bf16x8 V8;
   typedef __bf16 V2 __attribute__((ext_vector_type(2)));
   static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  // position-fixed forms: accumulator in VGPRs with operands from AGPRs, and the other way round.  The compiler
+  // does not see an MFMA in the asm statement, so the wait states a preceding VALU/AGPR write of an operand
+  // needs are supplied here.
+  static __device__ __forceinline__ void mma_v(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "a"(a), "a"(b)); }
+  static __device__ __forceinline__ void mma_v_first(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(acc) : "a"(a), "a"(b)); }
+  static __device__ __forceinline__ void mma_a(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b)); }
   static __device__ __forceinline__ float dot_ones(V2 a, float acc) {
     V2 one;
     one[0] = (__bf16)1.0f;
@@ -52,6 +58,9 @@ template <> struct Mma<f16_t> {
   typedef f16x8 V8;
   typedef _Float16 V2 __attribute__((ext_vector_type(2)));
   static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ void mma_v(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "a"(a), "a"(b)); }
+  static __device__ __forceinline__ void mma_v_first(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(acc) : "a"(a), "a"(b)); }
+  static __device__ __forceinline__ void mma_a(f32x16& acc, V8 a, V8 b) { asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b)); }
   static __device__ __forceinline__ float dot_ones(V2 a, float acc) {
     V2 one;
     one[0] = (_Float16)1.0f;
@@ -240,47 +249,43 @@ __global__ __launch_bounds__(256, 1) void select_pipe_kernel(AttnParams p, int n
     load_v(vbuf, v_start);
     const float mneg[2] = {-m_i[0], -m_i[1]};
 
-    // A(i+1): S^T of the next tile, accumulators taken round-robin
-    static_for<16>([&](auto j_tag) {
-      constexpr int j = decltype(j_tag)::value;
-      constexpr int ks = j >> 2, qt = (j >> 1) & 1, kt = j & 1;
-      if constexpr (ks == 0) {
-        f32x16 z;
+    // 32 slots, each: one MFMA, then the exponentials of two scores of the current tile.  Empty volatile asm
+    // statements on the score tuple before and on the probability tuple after pin the VALU instructions of the
+    // slot; a scheduling barrier after every slot keeps the MFMAs where they are written.
+    static_for<32>([&](auto s_tag) {
+      constexpr int s = decltype(s_tag)::value;
+      constexpr int j = s >> 1;
+      if constexpr ((s & 1) == 0) {  // A(i+1): S^T of the next tile, accumulators (VGPRs) taken round-robin
+        constexpr int ks = j >> 2, qt = (j >> 1) & 1, kt = j & 1;
+        if constexpr (ks == 0) {
+          f32x16 z;
 #pragma unroll
-        for (int r = 0; r < 16; r++) z[r] = 0.f;
-        st[OTH][qt][kt] = Mma<E>::mma(ak[OTH][kt][ks], bq[qt][ks], z);
-      } else {
-        st[OTH][qt][kt] = Mma<E>::mma(ak[OTH][kt][ks], bq[qt][ks], st[OTH][qt][kt]);
+          for (int r = 0; r < 16; r++) z[r] = 0.f;
+          st[OTH][qt][kt] = Mma<E>::mma(ak[OTH][kt][ks], bq[qt][ks], z);
+        } else {
+          st[OTH][qt][kt] = Mma<E>::mma(ak[OTH][kt][ks], bq[qt][ks], st[OTH][qt][kt]);
+        }
+      } else {  // C(i-1): PV of the previous tile into the AGPR accumulators
+        constexpr int kj = j >> 2, dt = (j >> 1) & 1, qt = j & 1;
+        constexpr int kt = kj >> 1, jj = kj & 1;
+        ot[dt][qt] = Mma<E>::mma(vfr[kt][jj][dt], pf[OTH][qt][kt][jj], ot[dt][qt]);
       }
+      {  // B(i): element pair e, e+1 of the current tile
+        constexpr int e = 2 * s;
+        constexpr int qt = e >> 5, kt = (e >> 4) & 1, r = e & 15, jj = r >> 3, e8 = r & 7;
+        asm volatile("" : "+v"(st[PAR][qt][kt]));
+        const float x0 = __builtin_amdgcn_exp2f(fmaf(st[PAR][qt][kt][r], sl2, mneg[qt]));
+        const float x1 = __builtin_amdgcn_exp2f(fmaf(st[PAR][qt][kt][r + 1], sl2, mneg[qt]));
+        V2 pk;
+        pk[0] = (E)x0;
+        pk[1] = (E)x1;
+        pf[PAR][qt][kt][jj][e8] = pk[0];
+        pf[PAR][qt][kt][jj][e8 + 1] = pk[1];
+        l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
+        asm volatile("" : "+v"(pf[PAR][qt][kt][jj]), "+v"(l_i[qt]));
+      }
+      __builtin_amdgcn_sched_barrier(0);
     });
-    // C(i-1): PV of the previous tile
-    static_for<16>([&](auto j_tag) {
-      constexpr int j = decltype(j_tag)::value;
-      constexpr int kj = j >> 2, dt = (j >> 1) & 1, qt = j & 1;
-      constexpr int kt = kj >> 1, jj = kj & 1;
-      ot[dt][qt] = Mma<E>::mma(vfr[kt][jj][dt], pf[OTH][qt][kt][jj], ot[dt][qt]);
-    });
-    // B(i): element pair pr = (qt, kt, r = 2*(pr%8), 2*(pr%8)+1)
-    static_for<32>([&](auto pr_tag) {
-      constexpr int e = 2 * decltype(pr_tag)::value;
-      constexpr int qt = e >> 5, kt = (e >> 4) & 1, r = e & 15, jj = r >> 3, e8 = r & 7;
-      const float x0 = __builtin_amdgcn_exp2f(fmaf(st[PAR][qt][kt][r], sl2, mneg[qt]));
-      const float x1 = __builtin_amdgcn_exp2f(fmaf(st[PAR][qt][kt][r + 1], sl2, mneg[qt]));
-      V2 pk;
-      pk[0] = (E)x0;
-      pk[1] = (E)x1;
-      pf[PAR][qt][kt][jj][e8] = pk[0];
-      pf[PAR][qt][kt][jj][e8 + 1] = pk[1];
-      l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
-    });
-  };
-  // scheduling pattern for one iteration: one MFMA, then six of the 192 VALU instructions of the softmax
-  auto interleave = [&]() {
-#pragma unroll
-    for (int s = 0; s < 32; s++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-    }
   };
   // PV of a finished probability tile without anything to overlap it with
   auto pv_only = [&](const V8 (&pp)[2][2][2], int buf) {
@@ -409,21 +414,20 @@ __global__ __launch_bounds__(256, 1) void select_pipe_kernel(AttnParams p, int n
     int i = 0;
     for (int pr = n_full >> 1; pr > 0; pr--) {  // two iterations per trip, no branch inside
       iteration(std::integral_constant<int, 0>{}, i == 0 ? 0 : (i - 1) & 3, k_next, v_next, (i + 1) & 3);
-      interleave();
       v_next = k_next;
       k_next = pop_or_last();
       i++;
       iteration(std::integral_constant<int, 1>{}, (i - 1) & 3, k_next, v_next, (i + 1) & 3);
-      interleave();
       v_next = k_next;
       k_next = pop_or_last();
       i++;
     }
     if (n_full & 1) {
       iteration(std::integral_constant<int, 0>{}, i == 0 ? 0 : (i - 1) & 3, k_next, v_next, (i + 1) & 3);
-      interleave();
+      asm volatile("s_nop 15\n\ts_nop 15");  // the asm MFMAs' results settle before compiler-scheduled code reads them
       pv_only(pf[0], (n_full - 1) & 3);
     } else {
+      asm volatile("s_nop 15\n\ts_nop 15");
       pv_only(pf[1], (n_full - 1) & 3);
     }
     // a reference that was too low shows up as a huge or non-finite row sum
