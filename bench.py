@@ -169,7 +169,7 @@ def main() -> int:
         "hbm_gbs": {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9, "merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9},
         "peak_mem_gb": peak_mem / 1e9,
         "roofline": {
-            "kernel": "select_mfma_kernel",
+            "kernel": "select_pipe_kernel",
             "bound": "mfma",
             "achieved": sel_tflops,
             "peak": PEAK_BF16_TFLOPS,

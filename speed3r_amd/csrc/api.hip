@@ -82,17 +82,17 @@ extern "C" int s3r_select_attn(const void* q, const void* k, const void* v, cons
   p.scale = softmax_scale;
 
   const int es = elt_size(dtype);
+  // (row strides below 2^20 elements: the tile transfers use 32-bit byte offsets inside a 64-row tile)
   const bool mfma_ok = dtype != S3R_F32 && D == 64 && block == 64 && K <= 64 && softmax_scale > 0.f &&
-                       vec_ok(q, es, sqb, sqh, sqn) && vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
+                       skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) && vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
                        vec_ok(o, es, sob, soh, son);
   if (mfma_ok) {
-    // S3R_SELECT_KERNEL=pipe picks the one-wave-per-SIMD software-pipelined kernel (currently the slower one:
-    // the compiler's schedule of its loop body clusters the MFMAs instead of interleaving them)
-    static const bool pipe = [] {
+    // default: the software-pipelined kernel; S3R_SELECT_KERNEL=basic picks the unpipelined one
+    static const bool basic = [] {
       const char* e = getenv("S3R_SELECT_KERNEL");
-      return e != nullptr && strcmp(e, "pipe") == 0;
+      return e != nullptr && strcmp(e, "basic") == 0;
     }();
-    return pipe ? launch_select_pipe(p, dtype, stream) : launch_select_mfma(p, dtype, stream);
+    return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
   }
   return launch_attn_simple(p, dtype, /*select=*/true, stream);
 }

@@ -33,63 +33,12 @@
 // Workgroup -> work mapping is XCD-aware: hardware deals workgroups round-robin over the 8
 // XCDs, so workgroup w is given work item (w % 8) * per_xcd + w / 8: each XCD then walks a
 // contiguous range of query blocks of one head at a time and its L2 sees one head's K/V.
-#include "s3r_common.h"
+#include "select_common.h"
 #include "attn_params.h"
-#include <type_traits>
-#include <utility>
 
 namespace s3r {
 namespace basic {
-
-template <typename E> struct Mma;
-template <> struct Mma<bf16_t> {
-  typedef bf16x8 V8;
-  typedef __bf16 V2 __attribute__((ext_vector_type(2)));
-  static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-  static __device__ __forceinline__ float dot_ones(V2 a, float acc) {
-    V2 one;
-    one[0] = (__bf16)1.0f;
-    one[1] = (__bf16)1.0f;
-    return __builtin_amdgcn_fdot2_f32_bf16(a, one, acc, false);
-  }
-};
-template <> struct Mma<f16_t> {
-  typedef f16x8 V8;
-  typedef _Float16 V2 __attribute__((ext_vector_type(2)));
-  static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-  static __device__ __forceinline__ float dot_ones(V2 a, float acc) {
-    V2 one;
-    one[0] = (_Float16)1.0f;
-    one[1] = (_Float16)1.0f;
-    return __builtin_amdgcn_fdot2(a, one, acc, false);
-  }
-};
-
-union Frag {
-  uint4 u;
-  bf16x8 b;
-  f16x8 h;
-  s16x4 s[2];
-};
-template <typename E> __device__ __forceinline__ typename Mma<E>::V8 as_v8(const Frag& f);
-template <> __device__ __forceinline__ bf16x8 as_v8<bf16_t>(const Frag& f) { return f.b; }
-template <> __device__ __forceinline__ f16x8 as_v8<f16_t>(const Frag& f) { return f.h; }
-
-__device__ __forceinline__ float xh_max(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float xh_sum(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
-}
+using namespace sel;
 
 constexpr int kTile = 64 * 64;  // elements per LDS tile buffer (one K and one V buffer per wave)
 
@@ -206,6 +155,9 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
     for (int i = 0; i < 8; i++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(kl + i * 512), 16, klds_off, i * k_step, 0, 0);
   };
+  // Every read of a tile buffer is preceded by an explicit wait for its transfer (the compiler's own bookkeeping of
+  // transfers into LDS is not relied on): vmcnt counts in issue order and K and V transfers alternate, 8 instructions each.
+  auto wait_transfer = [&]() { __builtin_amdgcn_s_waitcnt(0x0F78); };  // vmcnt(8)
   const int kr_off = c * 128 + ((hh ^ (c & 7)) << 4);
   auto read_k = [&](V8 (&dst)[2][4]) {
     const char* kbase = reinterpret_cast<const char*>(kl);
@@ -285,6 +237,7 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
   // buffer is free from then on) and that of the next V tile after the PV reads: each has about one tile of time.
   auto fast_tile = [&](int64_t next) {
     const float mneg[2] = {-m_i[0], -m_i[1]};
+    wait_transfer();
     read_k(ak[0]);
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
@@ -315,7 +268,9 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
           }
     }
     __builtin_amdgcn_sched_barrier(0);
+    wait_transfer();
     pv_only(pf[0]);
+    __builtin_amdgcn_sched_barrier(0);  // the refill is issued after the MFMAs that consumed the old contents
     load_v(next);
   };
   // Unpipelined stage with a true online softmax: one key tile (possibly ragged) from global memory.
@@ -402,6 +357,7 @@ __global__ __launch_bounds__(256, 2) void select_mfma_kernel(AttnParams p, int n
       last_start = any ? s : last_start;
       return last_start;
     };
+    wait_transfer();
     read_k(ak[0]);
     scores_only(st[0], ak[0]);
     m_i[0] = row_max(st[0][0]);
