@@ -37,7 +37,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
-    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge"],
+    ap.add_argument("--no-fuse-merge", action="store_true", help="run selection attention and the gated merge as two kernels")
+    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
 
@@ -85,7 +86,8 @@ def main() -> int:
     qd, kd, vd, gd = (t.to(dev) for t in (q, k, v, gate))
     mat = True if args.materialize_scores else None
 
-    names = ["pool", "compressed_topk", "select", "merge"]
+    fused = not args.no_fuse_merge
+    names = ["pool", "compressed_topk", "select_merge"] if fused else ["pool", "compressed_topk", "select", "merge"]
 
     def step(events=None):
         def mark(i):
@@ -96,6 +98,11 @@ def main() -> int:
         mark(1)
         o_cmp, idx = s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat)
         mark(2)
+        if fused:   # the merge runs in the selection kernel's epilogue (same bits as the two kernels)
+            out = s3r.select_attn_merge(qd, kd, vd, idx, o_cmp, gd, block)
+            assert out is not None, "the library has no fused selection+merge kernel for this shape"
+            mark(3)
+            return out
         o_sel = s3r.select_attn(qd, kd, vd, idx, block)
         mark(3)
         out = s3r.gated_merge(o_cmp, o_sel, gd, block)
@@ -112,6 +119,7 @@ def main() -> int:
                 "compressed_topk": lambda: s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat),
                 "select": lambda: s3r.select_attn(qd, kd, vd, idx, block),
                 "merge": lambda: s3r.gated_merge(o_cmp, o_sel, gd, block),
+                "select_merge": lambda: s3r.select_attn_merge(qd, kd, vd, idx, o_cmp, gd, block),
             }[args.only]
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -139,7 +147,8 @@ def main() -> int:
     kern_ms = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
     f_sel = workloads.selection_flops(n, topk)
     f_cmp = workloads.compressed_flops(n)
-    sel_tflops = f_sel / (kern_ms["select"] * 1e-3) / 1e12
+    sel_name = "select_merge" if fused else "select"
+    sel_tflops = f_sel / (kern_ms[sel_name] * 1e-3) / 1e12
     es = 2 if cfg.dtype != torch.float32 else 4
     pool_bytes = 3 * (n + nc) * 16 * 64 * es
     merge_bytes = (2 * n * 16 * 64 + n * 16 * 2 + nc * 16 * 64) * es
@@ -166,10 +175,11 @@ def main() -> int:
         },
         "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
         "kernels_ms": kern_ms,
-        "hbm_gbs": {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9, "merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9},
+        "hbm_gbs": {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9,
+                    **({} if fused else {"merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9})},
         "peak_mem_gb": peak_mem / 1e9,
         "roofline": {
-            "kernel": "select_pipe_kernel",
+            "kernel": "select_pipe_kernel" + (" (gated merge in its epilogue)" if fused else ""),
             "bound": "mfma",
             "achieved": sel_tflops,
             "peak": PEAK_BF16_TFLOPS,

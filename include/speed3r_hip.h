@@ -109,6 +109,29 @@ int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* 
                     float softmax_scale, int dtype, void* stream);
 
 /*
+ * Selection-branch attention with the gated merge in its epilogue: the selection output never
+ * goes to memory; the kernel writes
+ *   out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d]
+ * with the rounding points of s3r_gated_merge (o_sel, each product and the sum rounded to the I/O
+ * dtype), so the result equals s3r_select_attn followed by s3r_gated_merge bit for bit.
+ * Replaces topk_blocksparse_attention (pi3/models/sparse_attn/topk_blocksparse_attention.py:1093-1121)
+ * together with the merge expression of pi3/models/layers/sparse_attention.py:127-136.
+ * Arguments as in s3r_select_attn and s3r_gated_merge; out is contiguous [B,N,H*D].
+ * Only for the MFMA path (bf16/fp16, D == 64, block == 64, 16-byte aligned tensors); other
+ * shapes return S3R_ERR_UNSUPPORTED and the caller runs the two operators one after the other.
+ */
+int s3r_select_attn_merge(const void* q, const void* k, const void* v, const int32_t* idx,
+                          const void* o_cmp, const void* gate, void* out,
+                          int B, int H, int64_t N, int D, int block, int K,
+                          int64_t sqb, int64_t sqh, int64_t sqn,
+                          int64_t skb, int64_t skh, int64_t skn,
+                          int64_t svb, int64_t svh, int64_t svn,
+                          int64_t sib, int64_t sih, int64_t sim,
+                          int64_t scb, int64_t sch, int64_t scm,
+                          int64_t sgb, int64_t sgh, int64_t sgn,
+                          float softmax_scale, int dtype, void* stream);
+
+/*
  * Gated merge of the two branches, written in the [B,N,H*D] layout the output projection
  * reads:  out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d].
  * Replaces the einops/broadcast expression in pi3/models/layers/sparse_attention.py:127-136.

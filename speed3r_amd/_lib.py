@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libspeed3r_hip.so"
 
 S3R_F32, S3R_BF16, S3R_F16 = 0, 1, 2
 S3R_OK = 0
+S3R_ERR_BAD_ARG, S3R_ERR_UNSUPPORTED, S3R_ERR_HIP = -1, -2, -3
 
 # name -> (restype, argtypes); mirrors include/speed3r_hip.h declaration by declaration
 _i64x3 = [c_int64, c_int64, c_int64]
@@ -28,6 +29,9 @@ SIGNATURES = {
     "s3r_select_attn": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_int, c_int, c_int64, c_int, c_int, c_int,
                                 *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
+    "s3r_select_attn_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_int, c_int64, c_int, c_int, c_int,
+                                      *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
     "s3r_gated_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int,
                                 *_i64x3, *_i64x3, *_i64x3, c_int, c_void_p]),
 }

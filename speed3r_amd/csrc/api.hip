@@ -61,17 +61,30 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
   return rc;
 }
 
-extern "C" int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx, void* o, float* lse,
-                               int B, int H, int64_t N, int D, int block, int K,
-                               int64_t sqb, int64_t sqh, int64_t sqn, int64_t skb, int64_t skh, int64_t skn,
-                               int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t son,
-                               int64_t sib, int64_t sih, int64_t sim, float softmax_scale, int dtype, void* stream) {
-  if (!q || !k || !v || !idx || !o) return fail(S3R_ERR_BAD_ARG, "s3r_select_attn: null pointer");
-  if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || K <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_select_attn: non-positive size");
-  if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: dtype %d", dtype);
-  if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: head_dim %d > 64", D);
+namespace s3r {
+
+// merge arguments of the fused variant; out == nullptr: plain selection attention
+struct MergeArgs {
+  const void* o_cmp;
+  const void* gate;
+  void* out;
+  int64_t scb, sch, scm, sgb, sgh, sgn;
+};
+
+static int select_attn_impl(const char* who, const void* q, const void* k, const void* v, const int32_t* idx, void* o, float* lse,
+                            int B, int H, int64_t N, int D, int block, int K,
+                            int64_t sqb, int64_t sqh, int64_t sqn, int64_t skb, int64_t skh, int64_t skn,
+                            int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t son,
+                            int64_t sib, int64_t sih, int64_t sim, float softmax_scale, int dtype, const MergeArgs& m,
+                            void* stream) {
+  const bool merge = m.out != nullptr;
+  if (!q || !k || !v || !idx || (!merge && !o)) return fail(S3R_ERR_BAD_ARG, "%s: null pointer", who);
+  if (merge && (!m.o_cmp || !m.gate)) return fail(S3R_ERR_BAD_ARG, "%s: null pointer", who);
+  if (B <= 0 || H <= 0 || N <= 0 || D <= 0 || K <= 0) return fail(S3R_ERR_BAD_ARG, "%s: non-positive size", who);
+  if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+  if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "%s: head_dim %d > 64", who, D);
   if (block != 4 && block != 16 && block != 32 && block != 64)
-    return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: block %d not in {4,16,32,64}", block);
+    return fail(S3R_ERR_UNSUPPORTED, "%s: block %d not in {4,16,32,64}", who, block);
 
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.scores = nullptr; p.idx = idx; p.topk_idx = nullptr;
@@ -80,19 +93,51 @@ extern "C" int s3r_select_attn(const void* q, const void* k, const void* v, cons
   p.svb = svb; p.svh = svh; p.svn = svn; p.sob = sob; p.soh = soh; p.som = son;
   p.sib = sib; p.sih = sih; p.sim = sim;
   p.scale = softmax_scale;
+  p.merge_oc = m.o_cmp; p.merge_gate = m.gate; p.merge_out = m.out;
+  p.scb = m.scb; p.sch = m.sch; p.scm = m.scm; p.sgb = m.sgb; p.sgh = m.sgh; p.sgn = m.sgn;
 
   const int es = elt_size(dtype);
   // (row strides below 2^20 elements: the tile transfers use 32-bit byte offsets inside a 64-row tile)
   const bool mfma_ok = dtype != S3R_F32 && D == 64 && block == 64 && K <= 64 && softmax_scale > 0.f &&
-                       skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) && vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
-                       vec_ok(o, es, sob, soh, son);
-  if (mfma_ok) {
-    // default: the software-pipelined kernel; S3R_SELECT_KERNEL=basic picks the unpipelined one
-    static const bool basic = [] {
-      const char* e = getenv("S3R_SELECT_KERNEL");
-      return e != nullptr && strcmp(e, "basic") == 0;
-    }();
-    return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
+                       skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
+                       vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
+                       (merge ? (vec_ok(m.o_cmp, es, m.scb, m.sch, m.scm) && aligned16(m.out)) : vec_ok(o, es, sob, soh, son));
+  // default: the software-pipelined kernel; S3R_SELECT_KERNEL=basic picks the unpipelined one
+  static const bool basic = [] {
+    const char* e = getenv("S3R_SELECT_KERNEL");
+    return e != nullptr && strcmp(e, "basic") == 0;
+  }();
+  if (merge) {
+    if (!mfma_ok || basic)
+      return fail(S3R_ERR_UNSUPPORTED, "%s: the fused merge needs the pipelined MFMA kernel (bf16/fp16, head_dim 64, block 64, "
+                                       "16-byte aligned tensors); run s3r_select_attn and s3r_gated_merge instead", who);
+    return launch_select_pipe(p, dtype, stream);
   }
+  if (mfma_ok) return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
   return launch_attn_simple(p, dtype, /*select=*/true, stream);
+}
+
+}  // namespace s3r
+
+extern "C" int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx, void* o, float* lse,
+                               int B, int H, int64_t N, int D, int block, int K,
+                               int64_t sqb, int64_t sqh, int64_t sqn, int64_t skb, int64_t skh, int64_t skn,
+                               int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t son,
+                               int64_t sib, int64_t sih, int64_t sim, float softmax_scale, int dtype, void* stream) {
+  const MergeArgs none = {};
+  return select_attn_impl("s3r_select_attn", q, k, v, idx, o, lse, B, H, N, D, block, K, sqb, sqh, sqn, skb, skh, skn,
+                          svb, svh, svn, sob, soh, son, sib, sih, sim, softmax_scale, dtype, none, stream);
+}
+
+extern "C" int s3r_select_attn_merge(const void* q, const void* k, const void* v, const int32_t* idx,
+                                     const void* o_cmp, const void* gate, void* out,
+                                     int B, int H, int64_t N, int D, int block, int K,
+                                     int64_t sqb, int64_t sqh, int64_t sqn, int64_t skb, int64_t skh, int64_t skn,
+                                     int64_t svb, int64_t svh, int64_t svn, int64_t sib, int64_t sih, int64_t sim,
+                                     int64_t scb, int64_t sch, int64_t scm, int64_t sgb, int64_t sgh, int64_t sgn,
+                                     float softmax_scale, int dtype, void* stream) {
+  if (!out) return fail(S3R_ERR_BAD_ARG, "s3r_select_attn_merge: null pointer");
+  const MergeArgs m = {o_cmp, gate, out, scb, sch, scm, sgb, sgh, sgn};
+  return select_attn_impl("s3r_select_attn_merge", q, k, v, idx, nullptr, nullptr, B, H, N, D, block, K, sqb, sqh, sqn,
+                          skb, skh, skn, svb, svh, svn, 0, 0, 0, sib, sih, sim, softmax_scale, dtype, m, stream);
 }

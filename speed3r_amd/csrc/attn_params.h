@@ -22,6 +22,13 @@ struct AttnParams {
   int64_t sob, soh, som;
   int64_t sib, sih, sim;
   float scale;
+  // selection branch with fused gated merge (merge_out != nullptr): instead of o the kernel writes
+  // merge_out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d]  (contiguous [B,Lq,H*D])
+  const void* merge_oc;
+  const void* merge_gate;
+  void* merge_out;
+  int64_t scb, sch, scm;
+  int64_t sgb, sgh, sgn;
 };
 
 // launchers implemented in the .hip files; each returns S3R_OK or an error code

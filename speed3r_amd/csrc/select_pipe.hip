@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   uint64_t todo = __ballot(my_valid && my_idx != ragged_blk);
   int n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
   const int n_full = __popcll(todo);
-  if (n_full + n_ragged == 0) {
+  if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
       const int64_t row = q0 + qt * 32 + c;
@@ -422,24 +422,61 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   }
   for (; n_ragged > 0; n_ragged--) robust_tile((int64_t)ragged_blk * 64);
 
+  // Output: lane (c, hh) holds for query c + 32*qt the head_dim values dt*32 + 8*g4 + 4*hh + {0..3}.  One exchange with
+  // lane ^ 32 per packed word hands every lane eight consecutive head_dim values (hh = 0: group g4 = 2*gp, hh = 1:
+  // group 2*gp + 1), so a row receives 32 contiguous bytes per store instruction.
+  const bool merge = p.merge_out != nullptr;
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
+#pragma clang fp contract(off)  // the merge rounds each product and the sum separately, like the eager expression
     const float l = xh_sum(l_i[qt]);
     const float inv = l > 0.f ? 1.f / l : 0.f;
     const int64_t row = q0 + qt * 32 + c;
-    if (row < N) {
-#pragma unroll
-      for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-          union { E e[4]; uint2 u; } pk;
-#pragma unroll
-          for (int e = 0; e < 4; e++) pk.e[e] = (E)(ot[dt][qt][4 * g4 + e] * inv);
-          *reinterpret_cast<uint2*>(op + row * p.som + dt * 32 + 4 * hh + 8 * g4) = pk.u;
-        }
-      if (p.lse != nullptr && hh == 0)
-        p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+    const bool live = row < N;
+    float g0 = 0.f, g1 = 0.f;
+    if (merge && live) {
+      const E* gp = (const E*)p.merge_gate + (int64_t)b * p.sgb + (int64_t)h * p.sgh + row * p.sgn;
+      g0 = (float)gp[0];
+      g1 = (float)gp[1];
     }
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int gp = 0; gp < 2; gp++) {
+        union { E e[8]; uint32_t w[4]; uint4 u; } pc;
+        union { E e[2]; uint32_t w; } t;
+        uint32_t a[2], bw[2];
+#pragma unroll
+        for (int wi = 0; wi < 2; wi++) {
+          t.e[0] = (E)(ot[dt][qt][8 * gp + 2 * wi] * inv);
+          t.e[1] = (E)(ot[dt][qt][8 * gp + 2 * wi + 1] * inv);
+          a[wi] = t.w;
+          t.e[0] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi] * inv);
+          t.e[1] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi + 1] * inv);
+          bw[wi] = t.w;
+          const auto r = __builtin_amdgcn_permlane32_swap(a[wi], bw[wi], false, false);
+          pc.w[wi] = r[0];
+          pc.w[2 + wi] = r[1];
+        }
+        const int d0 = dt * 32 + 8 * (2 * gp + hh);
+        if (live) {
+          if (!merge) {
+            *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
+          } else {
+            union { E e[8]; uint4 u; } oc, res;
+            oc.u = *reinterpret_cast<const uint4*>((const E*)p.merge_oc + (int64_t)b * p.scb + (int64_t)h * p.sch + (int64_t)qb * p.scm + d0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const float x = round_to<E>(g0 * (float)oc.e[e]);
+              const float y = round_to<E>(g1 * (float)pc.e[e]);
+              res.e[e] = (E)(x + y);
+            }
+            *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = res.u;
+          }
+        }
+      }
+    if (live && p.lse != nullptr && hh == 0)
+      p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
   }
 }
 

@@ -199,14 +199,55 @@ def gated_merge(o_cmp: torch.Tensor, o_sel: torch.Tensor, gate: torch.Tensor, bl
     return out
 
 
+def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, o_cmp: torch.Tensor,
+                      gate: torch.Tensor, block: int, softmax_scale: Optional[float] = None) -> Optional[torch.Tensor]:
+    """``select_attn`` with ``gated_merge`` in its epilogue -> ``[B,N,H*D]``; bit-identical to the two calls, without the
+    round trip of the selection output through memory.  Returns ``None`` when the library has no fused kernel for the
+    shape (the caller then runs the two operators)."""
+    _need_device(q, k, v, idx, o_cmp, gate)
+    _forward_only(q, k, v, o_cmp, gate)
+    q, k, v, idx, o_cmp, gate = (_last_contig(t) for t in (q, k, v, idx, o_cmp, gate))
+    assert q.dtype == k.dtype == v.dtype == o_cmp.dtype == gate.dtype, "q, k, v, o_cmp, gate must share a dtype"
+    assert idx.dtype == torch.int32, "topk_idx must be int32"
+    b, h, n, d = q.shape
+    assert k.shape == q.shape and v.shape == q.shape, "q, k, v must share a shape"
+    nqb = -(-n // block)
+    assert idx.shape[:3] == (b, h, nqb), f"topk_idx shape {tuple(idx.shape)} does not match {(b, h, nqb, 'K')}"
+    assert o_cmp.shape == (b, h, nqb, d), f"o_cmp shape {tuple(o_cmp.shape)} != {(b, h, nqb, d)}"
+    assert gate.shape == (b, h, n, 2), f"gate shape {tuple(gate.shape)} != {(b, h, n, 2)}"
+    if q.dtype == torch.float32 or d != 64 or block != 64 or idx.shape[3] > 64:
+        return None
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    out = torch.empty((b, n, h * d), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().s3r_select_attn_merge(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), idx.data_ptr(), o_cmp.data_ptr(), gate.data_ptr(), out.data_ptr(),
+            b, h, n, d, block, idx.shape[3],
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), idx.stride(0), idx.stride(1), idx.stride(2),
+            o_cmp.stride(0), o_cmp.stride(1), o_cmp.stride(2), gate.stride(0), gate.stride(1), gate.stride(2),
+            scale, _code(q), _stream(q))
+    if rc == _lib.S3R_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "s3r_select_attn_merge")
+    return out
+
+
 def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
                             block: int = 64, topk: int = 16, softmax_scale: Optional[float] = None,
-                            return_parts: bool = False, materialize_scores: Optional[bool] = None):
+                            return_parts: bool = False, materialize_scores: Optional[bool] = None,
+                            fuse_merge: bool = True):
     """The whole path on post-norm/RoPE q, k, v ``[B,H,N,D]`` and gate ``[B,H,N,2]``:
     pool -> compressed attention + top-k -> selection attention -> gated merge -> ``[B,N,H*D]``.
+    The merge runs in the selection kernel's epilogue where the library offers it (same bits either way);
+    ``return_parts`` needs the selection output and therefore runs the two operators separately.
     """
     qc, kc, vc = pool_mean(q, block), pool_mean(k, block), pool_mean(v, block)
     o_cmp, idx = compressed_attn_topk(qc, kc, vc, topk, softmax_scale, materialize_scores=materialize_scores)
+    if fuse_merge and not return_parts:
+        out = select_attn_merge(q, k, v, idx, o_cmp, gate, block, softmax_scale)
+        if out is not None:
+            return out
     o_sel = select_attn(q, k, v, idx, block, softmax_scale)
     out = gated_merge(o_cmp, o_sel, gate, block)
     if return_parts:

@@ -199,6 +199,41 @@ def test_select_fixture(golden):
     assert max_abs(o, torch.from_numpy(golden["sel_out"])) <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,h,kk", [(256, 2, 2), (200, 3, 4), (1041, 2, 16), (64, 1, 1)])
+def test_select_with_fused_merge_equals_the_two_operators(dtype, n, h, kk):
+    """The merge in the selection kernel's epilogue must give the bits of select_attn followed by gated_merge
+    (ragged tail, skipped entries and empty rows included) and agree with the oracle's merge of the oracle's selection."""
+    b, d, block = 2, 64, 64
+    nqb = -(-n // block)
+    q, k, v = (_randn((b, h, n, d), 20 + i, dtype, 0.5).to(DEV) for i in range(3))
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randint(-1, nqb + 1, (b, h, nqb, kk), generator=g, dtype=torch.int32)   # -1 and nqb are skipped entries
+    idx[0, 0, 0, :] = -1                                                                  # an empty row
+    o_cmp = _randn((b, h, nqb, d), 30, dtype).to(DEV)
+    gate_lin = torch.sigmoid(_randn((b, n, 2 * h), 31, torch.float32)).to(dtype).to(DEV)
+    gate = gate_lin.view(b, n, h, 2).permute(0, 2, 1, 3)                                  # strided view, contiguous pair
+    o_sel = s3r.select_attn(q, k, v, idx.to(DEV), block)
+    want = s3r.gated_merge(o_cmp, o_sel, gate, block)
+    got = s3r.select_attn_merge(q, k, v, idx.to(DEV), o_cmp, gate, block)
+    assert got is not None and got.shape == (b, n, h * d)
+    assert torch.equal(got, want)
+    ref_sel = oracle.select_attention(q.cpu(), k.cpu(), v.cpu(), idx, block, out_dtype=torch.float32)
+    ref = oracle.gated_merge(o_cmp.cpu().float(), ref_sel, gate.cpu().float(), block)
+    assert max_abs(got, ref) <= 3e-2
+
+
+def test_fused_merge_declines_shapes_without_an_mfma_kernel():
+    b, h, n, d, block = 1, 2, 96, 64, 16
+    q, k, v = (_randn((b, h, n, d), 40 + i, torch.bfloat16).to(DEV) for i in range(3))
+    idx = torch.zeros((b, h, n // block, 2), dtype=torch.int32, device=DEV)
+    o_cmp = _randn((b, h, n // block, d), 43, torch.bfloat16).to(DEV)
+    gate = torch.rand((b, h, n, 2), dtype=torch.float32).to(torch.bfloat16).to(DEV)
+    assert s3r.select_attn_merge(q, k, v, idx, o_cmp, gate, block) is None
+    out = s3r.sparse_global_attention(q, k, v, gate, block=block, topk=2)      # falls back to the two operators
+    assert out.shape == (b, n, h * d)
+
+
 def test_select_empty_row_gives_zeros_and_strided_inputs_work():
     n, h = 256, 2
     qkv = _randn((1, n, 3, h, 64), 9, torch.bfloat16, 0.5).to(DEV)
