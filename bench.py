@@ -170,8 +170,7 @@ def main() -> int:
             "workload": f"{cfg.name}: {cfg.frames} frames x {workloads.TOKENS_PER_FRAME} tokens = {n} tokens, "
                         f"16 heads x 64, block {block}, top-k {topk}, B=1",
             "tokens": n, "heads": 16, "head_dim": 64, "block": block, "topk": topk,
-            "scores": "materialized" if (args.materialize_scores or 16 * nc * nc * 4 <= s3r.sparse_attn.ops.SCORE_BUFFER_LIMIT)
-                      else "fused",
+            "scores": "materialized" if args.materialize_scores else "fused (never leave the chip)",
         },
         "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
         "kernels_ms": kern_ms,

@@ -170,6 +170,19 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
       *reinterpret_cast<uint4*>(&Vs[buf][r * 64 + ld_pos * 8]) = vr[i];
     }
   };
+  // second pass of the fused selection: K tiles only, two per step (the second one of a pair lives in the V buffer)
+  auto fetch_kk = [&](int64_t start) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int r = ld_row + 32 * i;
+      int64_t row = start + r;
+      row = row < Lk ? row : Lk - 1;
+      kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
+      row = start + 64 + r;
+      row = row < Lk ? row : Lk - 1;
+      vr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
+    }
+  };
   // per-lane LDS read offsets (bytes)
   const int i16 = lane & 15;
   const int tr_row = 4 * hh + (i16 >> 2);
@@ -181,6 +194,7 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
 #pragma unroll
   for (int i = 0; i < KL; i++) list[i] = 0;
   float thr = __uint_as_float(0xFFFFFFFFu);  // a NaN: "s < thr" is false for every s, so everything passes
+  float thr0 = -INFINITY;                    // the row's threshold from the group maxima; thr never drops below it
   int qn = 0;
   uint2* qlane = FUSED ? &queue[wave][0][lane] : nullptr;  // entry e at qlane[e * 64]
   const uint32_t lkm1 = (uint32_t)(Lk - 1);
@@ -212,10 +226,16 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
     qn = 0;
     // threshold = score of the list's last entry (key 0, a filler, maps to a NaN: everything passes)
     const uint32_t k32 = (uint32_t)(list[KL - 1] >> 32);
-    thr = __uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu));
+    thr = fmaxf(__uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)), thr0);  // fmaxf drops the NaN
   };
 
   const int ntiles = (int)((Lk + 63) / 64);
+  // Fused selection, first pass: the maxima of the raw scores over groups of gsz key tiles (at most 128 groups per
+  // row) go to the wave's queue memory, which is idle until the second pass: gmax[group * 32 + row], as 16-bit
+  // floats (the upper half of the fp32 pattern) rounded DOWN, so that a threshold taken from them is still a lower bound.
+  const int gsz = (ntiles + 127) / 128;
+  uint16_t* gmax = FUSED ? reinterpret_cast<uint16_t*>(&queue[wave][0][0]) : nullptr;
+  float gm = -INFINITY;
   fetch(0);
   stash(0);
   if (ntiles > 1) fetch(64);
@@ -276,28 +296,6 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
     }
 
     const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
-    if constexpr (FUSED) {
-      // filter the raw scores against the lane's threshold; survivors go to the lane's queue
-      const uint32_t col0 = (uint32_t)start + 4 * hh;
-#pragma unroll
-      for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
-#pragma unroll
-        for (int e8 = 0; e8 < 8; e8++) {
-          const int kt = g >> 1, r = (g & 1) * 8 + e8;
-          const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
-          const float s = st[kt][r];
-          bool pass = !(s < thr);
-          if (partial) pass = pass && (koff < lim);
-          if (__any(pass)) {
-            uint2* dst = pass ? qlane + qn * 64 : qlane + (kQSlots - 1) * 64;  // non-survivors write the dump slot
-            *dst = make_uint2(__float_as_uint(s), col0 + koff);
-            qn += pass ? 1 : 0;
-          }
-        }
-        if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
-      }
-    }
-
     if (partial) {
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
@@ -311,6 +309,15 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
     mx = xh_max(mx);
+    if constexpr (FUSED) {
+      gm = fmaxf(gm, mx);
+      if ((t + 1) % gsz == 0 || t + 1 == ntiles) {
+        const uint32_t u = __float_as_uint(gm);
+        const uint32_t down = (u >> 16) + (((u >> 31) != 0 && (u & 0xffffu) != 0) ? 1u : 0u);  // negative: one step further down
+        if (hh == 0) gmax[(t / gsz) * 32 + c] = (uint16_t)down;
+        gm = -INFINITY;
+      }
+    }
     const float m_new = fmaxf(m_i, mx * sl2);
     const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
     float rowsum = 0.f;
@@ -368,6 +375,76 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
   }
 
   if constexpr (FUSED) {
+    // Threshold: the K-th largest group maximum of the row.  K different scores (one per group) are at least that
+    // large, so a score below it is not among the K largest, whatever the tie-break.  With fewer than K groups
+    // the threshold stays -inf and every score is a candidate.
+    {
+      float top[KL];
+#pragma unroll
+      for (int i = 0; i < KL; i++) top[i] = -INFINITY;
+      const int ngroups = (ntiles + gsz - 1) / gsz;
+      for (int g = 0; g < ngroups; g++) {
+        float x = __uint_as_float((uint32_t)gmax[g * 32 + c] << 16);
+#pragma unroll
+        for (int i = 0; i < KL; i++) {  // insertion into the descending list; NaN never enters (fmaxf/fminf drop it)
+          const float hi = fmaxf(top[i], x);
+          x = fminf(top[i], x);
+          top[i] = hi;
+        }
+      }
+      thr0 = qvalid ? top[KL - 1] : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
+      thr = thr0;
+    }
+    // Second pass: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
+    // through the lane's queue into its exact list.
+    __syncthreads();  // every wave is done with the tile buffers of the first pass (and with its own group maxima)
+    const int npairs = (ntiles + 1) / 2;
+    fetch_kk(0);
+    stash(0);
+    if (npairs > 1) fetch_kk(128);
+    for (int tp = 0; tp < npairs; tp++) {
+      const int buf = tp & 1;
+      __syncthreads();
+      if (tp + 1 < npairs) stash(buf ^ 1);
+      if (tp + 2 < npairs) fetch_kk((int64_t)(tp + 2) * 128);
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+        const int64_t start = (int64_t)tp * 128 + half * 64;
+        if (start >= Lk) break;  // odd number of tiles
+        const bool partial = start + 64 > Lk;
+        f32x16 st[2];
+        const char* kbase = reinterpret_cast<const char*>(half == 0 ? &Ks[buf][0] : &Vs[buf][0]);
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) {
+            Frag f;
+            f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
+            st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
+          }
+        }
+        const int lim = (int)(Lk - start) - 4 * hh;
+        const uint32_t col0 = (uint32_t)start + 4 * hh;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
+#pragma unroll
+          for (int e8 = 0; e8 < 8; e8++) {
+            const int kt = g >> 1, r = (g & 1) * 8 + e8;
+            const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
+            const float s = st[kt][r];
+            bool pass = !(s < thr);
+            if (partial) pass = pass && (koff < lim);
+            // no branch: every lane writes, non-survivors into the dump slot
+            uint2* dst = qlane + (pass ? qn : kQSlots - 1) * 64;
+            *dst = make_uint2(__float_as_uint(s), col0 + koff);
+            qn += pass ? 1 : 0;
+          }
+          if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
+        }
+      }
+    }
     drain();
     // the partner lane's list, then the K best of both, descending
     uint64_t other[KL];

@@ -17,7 +17,6 @@ import torch
 
 from .. import _lib
 
-SCORE_BUFFER_LIMIT = 4 << 30  # bytes of fp32 scores above which the fused selection is used by default
 
 _DTYPE_CODE = {torch.float32: _lib.S3R_F32, torch.bfloat16: _lib.S3R_BF16, torch.float16: _lib.S3R_F16}
 
@@ -88,9 +87,9 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk
 
     Returns ``(o, idx)`` with optional ``scores`` ([B,H,Lq,Lk] fp32) and ``lse`` appended when
     requested.  ``materialize_scores`` forces (True) or forbids (False) the fp32 score buffer.  By
-    default the scores go through HBM (attention kernel + row-wise top-k kernel, currently the faster
-    pair) while the buffer stays under ``SCORE_BUFFER_LIMIT`` bytes, and the selection is fused into
-    the attention kernel (scores never leave the chip) above that.
+    default the selection is fused into the attention kernel wherever the library has it (bf16/fp16,
+    head_dim 64, top-k a power of two up to 32): the scores never leave the chip.  Otherwise the scores
+    go through HBM (attention kernel, then the row-wise top-k kernel).
     """
     _need_device(q, k, v)
     _forward_only(q, k, v)
@@ -103,9 +102,8 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk
     o = torch.empty_like(q, memory_format=torch.contiguous_format)
     idx = torch.empty((b, h, lq, topk), dtype=torch.int32, device=q.device) if topk else None
     fused_ok = (q.dtype != torch.float32 and d == 64 and topk in (1, 2, 4, 8, 16, 32) and _lib.lib_has_fused_topk())
-    small = b * h * lq * lk * 4 <= SCORE_BUFFER_LIMIT
     want_scores = return_scores or (materialize_scores is True) or (
-        bool(topk) and materialize_scores is None and (small or not fused_ok))
+        bool(topk) and materialize_scores is None and not fused_ok)
     if materialize_scores is False and topk and not fused_ok:
         raise RuntimeError("fused top-k is not available for this dtype/shape; allow a score buffer")
     scores = torch.empty((b, h, lq, lk), dtype=torch.float32, device=q.device) if want_scores else None
