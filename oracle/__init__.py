@@ -18,3 +18,4 @@ from .sparse_attention_oracle import (  # noqa: F401
     gated_merge,
     sparse_global_attention,
 )
+from .sparse_layer_oracle import rope2d, block_positions, sparse_layer  # noqa: F401,E402

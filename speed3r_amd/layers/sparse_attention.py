@@ -1,0 +1,98 @@
+"""``SparseFlashAttentionRope``: the reference's global sparse attention layer
+(pi3/models/layers/sparse_attention.py:60-141) on the HIP kernels of this package.
+
+Same constructor arguments, same parameter names (``qkv``, ``proj``, ``q_norm``, ``k_norm``, ``gate.0``) and the
+same ``forward(x, attn_bias=None, xpos=None)``, so a reference checkpoint loads with ``load_state_dict``.
+Differences, all on the host side of the operator boundary:
+
+* q, k, v are handed to the kernels as strided views of the packed projection (no ``.contiguous()`` copies),
+  pooling reads the packed projection directly, and the gated merge runs in the selection kernel's epilogue
+  (or in its own kernel where that is not built), writing ``[B, N, C]`` for ``proj``;
+* forward only: run it under ``torch.no_grad()``;
+* ``N`` need not be a multiple of the block: the last block pools its valid tokens, its keys beyond ``N`` are
+  masked and its query rows beyond ``N`` do not exist (the reference raises for such ``N``);
+* the top-k count, 32 in the reference, is a constructor argument.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor, nn
+
+from ..sparse_attn import ops
+from ..sparse_attn.flash_attention_topk import flash_attn_topk_func
+from .pos_embed import block_positions
+
+
+class SparseFlashAttentionRope(nn.Module):
+    def __init__(
+        self,
+        dim: int,
+        num_heads: int = 16,
+        qkv_bias: bool = False,
+        proj_bias: bool = True,
+        attn_drop: float = 0.0,
+        proj_drop: float = 0.0,
+        qk_norm: bool = False,
+        norm_layer=nn.LayerNorm,
+        rope=None,
+        block_size: int = 4,
+        topk: int = 32,
+    ) -> None:
+        super().__init__()
+        assert dim % num_heads == 0, "dim must be a multiple of num_heads"
+        self.num_heads = num_heads
+        head_dim = dim // num_heads
+        self.scale = head_dim ** -0.5  # kept for parity with the reference; both operators default to it
+
+        self.qkv = nn.Linear(dim, dim * 3, bias=qkv_bias)
+        self.attn_drop = nn.Dropout(attn_drop)
+        self.proj = nn.Linear(dim, dim, bias=proj_bias)
+        self.proj_drop = nn.Dropout(proj_drop)
+        self.q_norm = norm_layer(head_dim) if qk_norm else nn.Identity()
+        self.k_norm = norm_layer(head_dim) if qk_norm else nn.Identity()
+        self.rope = rope
+
+        # gate: sigmoid(linear), weight 0 and bias (-1, +1) per head at initialisation
+        gate_linear = nn.Linear(dim, num_heads * 2, bias=True)
+        nn.init.zeros_(gate_linear.weight)
+        with torch.no_grad():
+            gate_linear.bias.copy_(torch.tensor([-1.0, 1.0]).repeat(num_heads))
+        self.gate = nn.Sequential(gate_linear, nn.Sigmoid())
+        self.block_size = block_size
+        self.topk = topk
+        self.keep_topk_idx = False   # debugging aid: keep the last forward's block indices in ``last_topk_idx``
+        self.last_topk_idx = None
+
+    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
+        b, n, c = x.shape
+        h = self.num_heads
+        d = c // h
+        block = self.block_size ** 2
+
+        qkv = self.qkv(x)                                              # [B, N, 3C], layout (qkv h d)
+        gate = self.gate(x).view(b, n, h, 2).permute(0, 2, 1, 3)       # [B, H, N, 2], strided view
+
+        # compressed branch: pooled raw projections -> norm -> RoPE at block positions -> attention + top-k
+        q_c, k_c, v_c = ops.pool_qkv_packed(qkv, h, block)
+        q_c, k_c = self.q_norm(q_c).to(v_c.dtype), self.k_norm(k_c).to(v_c.dtype)
+        if xpos is not None and self.rope is not None:
+            pos_c = block_positions(xpos, block)
+            q_c, k_c = self.rope(q_c, pos_c), self.rope(k_c, pos_c)
+        o_c, idx = flash_attn_topk_func(q_c, k_c, v_c, self.topk)
+        if self.keep_topk_idx:
+            self.last_topk_idx = idx
+
+        # selection branch on the full tokens (strided views of the projection; norm/RoPE make q, k contiguous)
+        q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)   # each [B, H, N, D]
+        q, k = self.q_norm(q).to(v.dtype), self.k_norm(k).to(v.dtype)
+        if xpos is not None and self.rope is not None:
+            q, k = self.rope(q, xpos), self.rope(k, xpos)
+
+        out = ops.select_attn_merge(q, k, v, idx, o_c, gate, block)
+        if out is None:
+            out = ops.gated_merge(o_c, ops.select_attn(q, k, v, idx, block), gate, block)
+
+        out = self.proj(out)
+        return self.proj_drop(out)
