@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
     ap.add_argument("--no-fuse-merge", action="store_true", help="run selection attention and the gated merge as two kernels")
-    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge"],
+    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "copy"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
 
@@ -120,6 +120,8 @@ def main() -> int:
                 "select": lambda: s3r.select_attn(qd, kd, vd, idx, block),
                 "merge": lambda: s3r.gated_merge(o_cmp, o_sel, gd, block),
                 "select_merge": lambda: s3r.select_attn_merge(qd, kd, vd, idx, o_cmp, gd, block),
+                # a plain device copy of q (reads and writes q.nbytes): the yardstick for the HBM byte counters
+                "copy": lambda: torch.empty_like(qd).copy_(qd),
             }[args.only]
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -184,7 +186,9 @@ def main() -> int:
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a plain copy (profiles/); measured for the
+            # default workload only
+            "traffic": 2.40e9 if (fused and args.config == "cfg3" and topk == 16) else None,
         },
     }
     if not args.no_cpu_baseline:
