@@ -194,6 +194,12 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
     return xh_max(mx) * sl2;
   };
+  auto half_max = [&](const f32x16& sc) -> float {  // over this lane's 16 keys of a half tile and its partner's
+    float mx = sc[0];
+#pragma unroll
+    for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
+    return xh_max(mx) * sl2;
+  };
   auto scores_half = [&](auto hf) {  // st[.][hf] from the K half in LDS
     constexpr int HF = decltype(hf)::value;
     read_k(hf, ak);
@@ -374,16 +380,14 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     dma_k(H1{}, s0);
     dma_v(H0{}, s0);
     int64_t s1 = pop_or_last(), s2 = pop_or_last();
-    // first tile: its row maxima become the softmax reference; st[.][0] stays for the first phase
+    // the row maxima over the first half tile become the softmax reference; st[.][0] stays for the first phase
     __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the first K half
     scores_half(H0{});
     reads_done();
     dma_k(H0{}, s1);  // the K half the second phase reads
     dma_v(H1{}, s0);
-    __builtin_amdgcn_s_waitcnt(0x0F7C);  // vmcnt(12): the second K half
-    scores_half(H1{});
-    m_i[0] = row_max(st[0]);
-    m_i[1] = row_max(st[1]);
+    m_i[0] = half_max(st[0][0]);
+    m_i[1] = half_max(st[1][0]);
     mneg[0] = -m_i[0];
     mneg[1] = -m_i[1];
 #pragma unroll
