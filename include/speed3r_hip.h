@@ -132,6 +132,25 @@ int s3r_select_attn_merge(const void* q, const void* k, const void* v, const int
                           float softmax_scale, int dtype, void* stream);
 
 /*
+ * qk-LayerNorm and 2-D rotary embedding of one [B,H,N,64] tensor (q or k) in one pass:
+ *   y = RoPE2D(LayerNorm(x) rounded to the I/O dtype, pos)
+ * Replaces self.q_norm / self.k_norm, the cast and self.rope of the reference layer
+ * (pi3/models/layers/sparse_attention.py:103-110,120-124) and RoPE2D.forward
+ * (pi3/models/layers/pos_embed.py:112-159).
+ *   x: strides sxb,sxh,sxn (last stride 1; the packed projection can be passed as a view); y: contiguous.
+ *   pos: int32 (y,x) per token, strides spb,spn (pair contiguous), or NULL for no rotation.
+ *   cos_tab, sin_tab: I/O dtype [P,16], row p = cos/sin of the angles p * base^(-2i/32), i = 0..15, with the
+ *     angles rounded to the I/O dtype first (the reference's table); positions are clamped to [0,P-1].
+ *   ln_w, ln_b: I/O dtype [64] LayerNorm weight and bias, ln_w NULL for no normalisation (ln_b optional).
+ * Products and sum of the rotation are rounded to the I/O dtype like the reference's eager expression.
+ */
+int s3r_norm_rope(const void* x, void* y, const int32_t* pos, const void* cos_tab, const void* sin_tab, int P,
+                  const void* ln_w, const void* ln_b, float eps,
+                  int B, int H, int64_t N, int D,
+                  int64_t sxb, int64_t sxh, int64_t sxn, int64_t spb, int64_t spn,
+                  int dtype, void* stream);
+
+/*
  * Gated merge of the two branches, written in the [B,N,H*D] layout the output projection
  * reads:  out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d].
  * Replaces the einops/broadcast expression in pi3/models/layers/sparse_attention.py:127-136.

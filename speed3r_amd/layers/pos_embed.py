@@ -14,10 +14,26 @@ from torch import nn
 
 
 class RoPE2D(nn.Module):
-    def __init__(self, freq: float = 100.0, F0: float = 1.0) -> None:
+    def __init__(self, freq: float = 100.0, F0: float = 1.0, max_positions: int = 0) -> None:
         super().__init__()
         self.base = freq
         self.F0 = F0
+        # number of rows of the cos/sin tables the fused kernel reads; 0: sized from the positions of every call
+        # (one device synchronisation per call, like the reference's ``positions.max()``)
+        self.max_positions = max_positions
+        self._tables = {}
+
+    def tables(self, head_dim: int, n_pos: int, device, dtype):
+        """cos, sin ``[n_pos, head_dim // 4]`` in ``dtype``: row p holds cos/sin of the angles ``p * inv_freq`` after
+        their rounding to ``dtype`` (the reference's table, pos_embed.py:121-131, without the duplicated half)."""
+        key = (head_dim, n_pos, str(device), dtype)
+        if key not in self._tables:
+            half = head_dim // 2
+            inv_freq = 1.0 / (self.base ** (torch.arange(0, half, 2, device=device, dtype=torch.float32) / half))
+            t = torch.arange(n_pos, device=device, dtype=torch.float32)
+            ang = torch.einsum("i,j->ij", t, inv_freq).to(dtype)
+            self._tables[key] = (ang.cos().contiguous(), ang.sin().contiguous())
+        return self._tables[key]
 
     def _cos_sin(self, pos1d: torch.Tensor, half: int, dtype: torch.dtype):
         # pos1d [B, N] integer coordinates -> cos, sin [B, 1, N, half] with the two quarters holding the same angles

@@ -22,7 +22,7 @@ from torch import Tensor, nn
 
 from ..sparse_attn import ops
 from ..sparse_attn.flash_attention_topk import flash_attn_topk_func
-from .pos_embed import block_positions
+from .pos_embed import RoPE2D, block_positions
 
 
 class SparseFlashAttentionRope(nn.Module):
@@ -65,6 +65,24 @@ class SparseFlashAttentionRope(nn.Module):
         self.keep_topk_idx = False   # debugging aid: keep the last forward's block indices in ``last_topk_idx``
         self.last_topk_idx = None
 
+    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
+        """qk-norm, cast and RoPE of one tensor: one fused kernel where it is built (head_dim 64, LayerNorm or no
+        norm, the package's RoPE2D), the separate torch modules otherwise.  Same rounding points either way."""
+        fused_norm = isinstance(norm, nn.Identity) or (type(norm) is nn.LayerNorm and norm.elementwise_affine)
+        fused_rope = pos is None or isinstance(self.rope, RoPE2D)
+        if t.shape[-1] == 64 and fused_norm and fused_rope and not (isinstance(norm, nn.Identity) and pos is None):
+            cos = sin = None
+            if pos is not None:
+                n_pos = self.rope.max_positions or int(pos.max()) + 1
+                cos, sin = self.rope.tables(64, n_pos, t.device, t.dtype)
+            ln = norm if isinstance(norm, nn.LayerNorm) else None
+            out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
+                                ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
+            if out is not None:
+                return out
+        t = norm(t).to(t.dtype)
+        return self.rope(t, pos) if pos is not None else t
+
     def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
         b, n, c = x.shape
         h = self.num_heads
@@ -76,19 +94,16 @@ class SparseFlashAttentionRope(nn.Module):
 
         # compressed branch: pooled raw projections -> norm -> RoPE at block positions -> attention + top-k
         q_c, k_c, v_c = ops.pool_qkv_packed(qkv, h, block)
-        q_c, k_c = self.q_norm(q_c).to(v_c.dtype), self.k_norm(k_c).to(v_c.dtype)
-        if xpos is not None and self.rope is not None:
-            pos_c = block_positions(xpos, block)
-            q_c, k_c = self.rope(q_c, pos_c), self.rope(k_c, pos_c)
+        pos_c = block_positions(xpos, block) if (xpos is not None and self.rope is not None) else None
+        q_c, k_c = self._norm_rope(q_c, self.q_norm, pos_c), self._norm_rope(k_c, self.k_norm, pos_c)
         o_c, idx = flash_attn_topk_func(q_c, k_c, v_c, self.topk)
         if self.keep_topk_idx:
             self.last_topk_idx = idx
 
         # selection branch on the full tokens (strided views of the projection; norm/RoPE make q, k contiguous)
         q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)   # each [B, H, N, D]
-        q, k = self.q_norm(q).to(v.dtype), self.k_norm(k).to(v.dtype)
-        if xpos is not None and self.rope is not None:
-            q, k = self.rope(q, xpos), self.rope(k, xpos)
+        pos = xpos if (xpos is not None and self.rope is not None) else None
+        q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
 
         out = ops.select_attn_merge(q, k, v, idx, o_c, gate, block)
         if out is None:

@@ -197,6 +197,44 @@ def gated_merge(o_cmp: torch.Tensor, o_sel: torch.Tensor, gate: torch.Tensor, bl
     return out
 
 
+def norm_rope(x: torch.Tensor, positions: Optional[torch.Tensor], cos_tab: Optional[torch.Tensor],
+              sin_tab: Optional[torch.Tensor], ln_weight: Optional[torch.Tensor] = None,
+              ln_bias: Optional[torch.Tensor] = None, eps: float = 1e-5) -> Optional[torch.Tensor]:
+    """``RoPE2D(LayerNorm(x), positions)`` for one ``[B,H,N,64]`` tensor in one pass -> contiguous ``[B,H,N,64]``.
+
+    ``positions``: integer ``[B,N,2]`` (or None: no rotation); ``cos_tab``/``sin_tab``: ``[P,16]`` tables in x's dtype
+    (``RoPE2D.tables``); ``ln_weight``/``ln_bias``: LayerNorm(64) parameters (None: no normalisation).
+    Returns None when the library has no kernel for the shape (head_dim other than 64)."""
+    _need_device(x)
+    _forward_only(x)
+    x = _last_contig(x)
+    b, h, n, d = x.shape
+    if d != 64:
+        return None
+    pos32 = None
+    p = 0
+    if positions is not None:
+        assert positions.shape == (b, n, 2), f"positions shape {tuple(positions.shape)} != {(b, n, 2)}"
+        assert cos_tab is not None and sin_tab is not None and cos_tab.shape == sin_tab.shape and cos_tab.shape[1] == 16
+        assert cos_tab.dtype == x.dtype and sin_tab.dtype == x.dtype, "tables must have x's dtype"
+        pos32 = positions.to(device=x.device, dtype=torch.int32).contiguous()
+        cos_tab, sin_tab = cos_tab.contiguous(), sin_tab.contiguous()
+        p = cos_tab.shape[0]
+    w = ln_weight.detach().to(x.dtype).contiguous() if ln_weight is not None else None
+    bias = ln_bias.detach().to(x.dtype).contiguous() if (ln_bias is not None and w is not None) else None
+    y = torch.empty((b, h, n, d), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().s3r_norm_rope(
+            x.data_ptr(), y.data_ptr(), pos32.data_ptr() if pos32 is not None else None,
+            cos_tab.data_ptr() if pos32 is not None else None, sin_tab.data_ptr() if pos32 is not None else None, p,
+            w.data_ptr() if w is not None else None, bias.data_ptr() if bias is not None else None, float(eps),
+            b, h, n, d, x.stride(0), x.stride(1), x.stride(2),
+            pos32.stride(0) if pos32 is not None else 0, pos32.stride(1) if pos32 is not None else 0,
+            _code(x), _stream(x))
+    _lib.check(rc, "s3r_norm_rope")
+    return y
+
+
 def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, o_cmp: torch.Tensor,
                       gate: torch.Tensor, block: int, softmax_scale: Optional[float] = None) -> Optional[torch.Tensor]:
     """``select_attn`` with ``gated_merge`` in its epilogue -> ``[B,N,H*D]``; bit-identical to the two calls, without the

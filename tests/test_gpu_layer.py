@@ -70,3 +70,37 @@ def test_layer_is_forward_only():
     x = torch.randn((1, 128, 128), device=DEV, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError):
         m(x)                      # parameters require grad and grad mode is on
+
+
+# ------------------------------------------------------------------------------------ fused qk-norm + RoPE kernel
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("with_norm,with_pos", [(True, True), (True, False), (False, True)])
+def test_norm_rope_kernel_matches_the_torch_modules(dtype, with_norm, with_pos):
+    """One pass of LayerNorm(64) + cast + RoPE2D against the separate torch modules on the same device, for a strided
+    view of a packed projection.  Same rounding points; the LayerNorm reduction order differs, so a few values may
+    land on the neighbouring representable number."""
+    import speed3r_amd as s3r
+    b, h, n, d = 2, 3, 333, 64
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn((b, n, 3 * h * d), generator=g).to(dtype).to(DEV)
+    x = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4)[1]                      # k as a strided [B,H,N,D] view
+    pos = torch.randint(0, 41, (b, n, 2), generator=g).to(DEV)
+    rope = RoPE2D(freq=100.0)
+    ln = torch.nn.LayerNorm(d, eps=1e-6).to(DEV)
+    with torch.no_grad():
+        ln.weight.uniform_(0.5, 1.5)
+        ln.bias.normal_(0, 0.1)
+    ln = ln.to(dtype)
+    cos, sin = rope.tables(d, 41, DEV, dtype)
+    with torch.no_grad():
+        got = s3r.sparse_attn.ops.norm_rope(x, pos if with_pos else None, cos if with_pos else None, sin if with_pos else None,
+                                            ln.weight if with_norm else None, ln.bias if with_norm else None, 1e-6)
+        want = ln(x).to(dtype) if with_norm else x
+        want = rope(want, pos) if with_pos else want
+    assert got.shape == (b, h, n, d) and got.is_contiguous()
+    tol = {torch.bfloat16: 4e-2, torch.float16: 5e-3, torch.float32: 1e-5}[dtype]
+    assert max_abs(got, want.float()) <= tol
+    if not with_norm:
+        assert torch.equal(got, want)                                              # no reduction involved: bit-identical
+    elif dtype != torch.float32:
+        assert (got == want).float().mean().item() >= 0.97
