@@ -32,7 +32,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
+                    help="cfg1-cfg4: one sparse global-attention layer call; cfg5: end-to-end Pi3_Sparse-style forward (frames/s)")
+    ap.add_argument("--frames", type=int, default=100, help="cfg5: number of 518x392 frames")
     ap.add_argument("--topk", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
@@ -65,6 +67,63 @@ def cpu_baseline(q, k, v, gate, block, topk, heads):
     }
 
 
+def run_end_to_end(args) -> int:
+    """cfg5: random-init Pi3_Sparse-style model, bf16, synthetic frames in [0,1]; frames/s and the share of GPU time
+    spent in the sparse global attention (HIP events around the 18 global attention modules)."""
+    import torch
+
+    from speed3r_amd.model import Pi3SparseLike
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(4)
+    model = Pi3SparseLike().to(torch.bfloat16).to(dev).eval()
+    g = torch.Generator().manual_seed(4)
+    imgs = torch.rand((1, args.frames, 3, 518, 392), generator=g).to(dev)
+    spans = []
+
+    def pre(_m, _a, _k=None):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        spans.append([e, None])
+
+    def post(_m, _a, _o):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        spans[-1][1] = e
+
+    for blk in model.global_decoder:
+        blk.attn.register_forward_pre_hook(pre)
+        blk.attn.register_forward_hook(post)
+    steps, warmup = min(args.steps, 5), min(args.warmup, 2)
+    with torch.no_grad():
+        for _ in range(max(warmup, 1)):
+            model(imgs)
+        torch.cuda.synchronize()
+        spans.clear()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = model(imgs)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    sparse_ms = sum(a.elapsed_time(b) for a, b in spans) / steps
+    ms = wall * 1e3 / steps
+    tokens = args.frames * 1041
+    print(json.dumps({
+        "metric": "frames/s, Pi3_Sparse-style forward (ViT-L/14 encoder + 36-layer decoder + heads), bf16",
+        "value": args.frames / (ms * 1e-3), "unit": "frames/s", "n_gpus": 1, "steps": steps, "warmup": max(warmup, 1),
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"cfg5: {args.frames} frames 518x392 -> {tokens} tokens (5 register + 1036 patch per frame), "
+                               "18 frame-local dense + 18 global sparse attention layers (block 64, top-k 16), random-init weights",
+                   "tokens": tokens, "block": 64, "topk": 16},
+        "sparse_attention_ms": sparse_ms, "sparse_attention_share": sparse_ms / ms,
+        "sparse_attention_ms_per_layer": sparse_ms / len(model.global_decoder),
+        "peak_mem_gb": torch.cuda.max_memory_allocated() / 1e9,
+        "outputs": {k: list(v.shape) for k, v in out.items()},
+    }))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -78,6 +137,8 @@ def main() -> int:
     from speed3r_amd import workloads
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    if args.config == "cfg5":
+        return run_end_to_end(args)
     dev = torch.device("cuda:0")
     cfg, q, k, v, gate = workloads.make_config(args.config)
     topk = args.topk or cfg.topk

@@ -1,0 +1,244 @@
+"""A Pi3_Sparse-style multi-view forward built around the package's sparse global attention layer.
+
+Purpose: the end-to-end throughput figure (frames/s, share of time in the sparse attention) of the reference's
+model family on random-initialised weights; it is not a weight-compatible re-implementation of the reference model.
+Structure after pi3/models/pi3_sparse.py:74-321 (encoder -> alternating frame-local / global decoder -> point,
+confidence and camera heads), pi3/models/layers/block.py:259-335 (pre-norm block with LayerScale),
+pi3/models/layers/transformer_head.py (head decoders, linear pixel-shuffle head):
+
+* patch encoder: ViT-L/14 with a class token and 4 register tokens (dim 1024, 24 blocks), dense attention per frame;
+* decoder: ``dec_depth // 2`` pairs of [frame-local dense attention block, global sparse attention block]
+  (dim 1024, 16 heads, MLP x4, qk-LayerNorm, LayerScale 0.01, RoPE2D base 100); the global block is
+  ``speed3r_amd.layers.SparseFlashAttentionRope`` over all frames' tokens;
+* tokens per frame: ``num_register`` register tokens followed by the patches in row-major order (the Pi3 teacher's
+  layout, pi3/models/pi3.py:140-154), so 518x392 frames give 5 + 37*28 = 1041 tokens; the global attention sees the
+  flat sequence in blocks of 64 tokens with the ragged-tail policy of the kernels;
+* heads: three 5-block frame-local decoders on the concatenated outputs of the last local and global blocks, a linear
+  pixel-shuffle head for local points and confidence, a small pose head.
+
+All dense GEMMs and the dense attentions are library calls (torch on rocBLAS/hipBLASLt, scaled_dot_product_attention).
+Inference only: call under ``torch.no_grad()`` with the module in one dtype (bf16).
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from ..layers import RoPE2D, SparseFlashAttentionRope
+from ..sparse_attn import ops
+
+
+class Mlp(nn.Module):
+    def __init__(self, dim: int, hidden: int) -> None:
+        super().__init__()
+        self.fc1 = nn.Linear(dim, hidden)
+        self.fc2 = nn.Linear(hidden, dim)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.fc2(F.gelu(self.fc1(x)))
+
+
+class LayerScale(nn.Module):
+    def __init__(self, dim: int, init_values: float) -> None:
+        super().__init__()
+        self.gamma = nn.Parameter(init_values * torch.ones(dim))
+
+    def forward(self, x: Tensor) -> Tensor:
+        return x * self.gamma
+
+
+class DenseAttentionRope(nn.Module):
+    """Dense attention inside each sequence of the batch (one frame), optional qk-norm and RoPE2D."""
+
+    def __init__(self, dim, num_heads=16, qkv_bias=True, proj_bias=True, attn_drop=0.0, proj_drop=0.0, qk_norm=False,
+                 norm_layer=nn.LayerNorm, rope=None) -> None:
+        super().__init__()
+        self.num_heads = num_heads
+        head_dim = dim // num_heads
+        self.qkv = nn.Linear(dim, dim * 3, bias=qkv_bias)
+        self.proj = nn.Linear(dim, dim, bias=proj_bias)
+        self.q_norm = norm_layer(head_dim) if qk_norm else nn.Identity()
+        self.k_norm = norm_layer(head_dim) if qk_norm else nn.Identity()
+        self.rope = rope
+
+    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
+        if t.is_cuda and t.shape[-1] == 64 and (pos is not None or isinstance(norm, nn.LayerNorm)):
+            cos = sin = None
+            if pos is not None:
+                cos, sin = self.rope.tables(64, self.rope.max_positions or int(pos.max()) + 1, t.device, t.dtype)
+            ln = norm if isinstance(norm, nn.LayerNorm) else None
+            out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
+                                ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
+            if out is not None:
+                return out
+        t = norm(t).to(t.dtype)
+        return self.rope(t, pos) if pos is not None else t
+
+    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
+        b, n, c = x.shape
+        h = self.num_heads
+        q, k, v = self.qkv(x).view(b, n, 3, h, c // h).permute(2, 0, 3, 1, 4).unbind(0)
+        pos = xpos if self.rope is not None else None
+        q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
+        o = F.scaled_dot_product_attention(q, k, v)
+        return self.proj(o.transpose(1, 2).reshape(b, n, c))
+
+
+class Block(nn.Module):
+    def __init__(self, dim, num_heads, attn_class, mlp_ratio=4.0, init_values=None, qk_norm=False, rope=None, **attn_kw):
+        super().__init__()
+        self.norm1 = nn.LayerNorm(dim, eps=1e-6)
+        self.attn = attn_class(dim, num_heads=num_heads, qkv_bias=True, proj_bias=True, qk_norm=qk_norm,
+                               norm_layer=partial(nn.LayerNorm, eps=1e-6), rope=rope, **attn_kw)
+        self.ls1 = LayerScale(dim, init_values) if init_values else nn.Identity()
+        self.norm2 = nn.LayerNorm(dim, eps=1e-6)
+        self.mlp = Mlp(dim, int(dim * mlp_ratio))
+        self.ls2 = LayerScale(dim, init_values) if init_values else nn.Identity()
+
+    def forward(self, x: Tensor, xpos: Optional[Tensor] = None) -> Tensor:
+        x = x + self.ls1(self.attn(self.norm1(x), xpos=xpos))
+        return x + self.ls2(self.mlp(self.norm2(x)))
+
+
+class PatchEncoder(nn.Module):
+    """ViT patch encoder: class token + register tokens + patch tokens with a learned position embedding."""
+
+    def __init__(self, dim=1024, depth=24, num_heads=16, patch=14, grid=(37, 28), num_register=4) -> None:
+        super().__init__()
+        self.patch = patch
+        self.grid = grid
+        self.patch_embed = nn.Conv2d(3, dim, kernel_size=patch, stride=patch)
+        self.cls_token = nn.Parameter(torch.zeros(1, 1, dim))
+        self.register_tokens = nn.Parameter(torch.zeros(1, num_register, dim))
+        self.pos_embed = nn.Parameter(torch.randn(1, 1 + grid[0] * grid[1], dim) * 0.02)
+        self.blocks = nn.ModuleList([Block(dim, num_heads, DenseAttentionRope, init_values=1e-5) for _ in range(depth)])
+        self.norm = nn.LayerNorm(dim, eps=1e-6)
+
+    def _pos(self, gh: int, gw: int) -> Tensor:
+        if (gh, gw) == self.grid:
+            return self.pos_embed
+        cls, patch = self.pos_embed[:, :1], self.pos_embed[:, 1:]
+        patch = patch.view(1, self.grid[0], self.grid[1], -1).permute(0, 3, 1, 2).float()
+        patch = F.interpolate(patch, size=(gh, gw), mode="bicubic", align_corners=False).to(self.pos_embed.dtype)
+        return torch.cat((cls, patch.permute(0, 2, 3, 1).reshape(1, gh * gw, -1)), dim=1)
+
+    def forward(self, imgs: Tensor) -> Tensor:  # [F,3,H,W] -> patch tokens [F, gh*gw, dim]
+        f = imgs.shape[0]
+        x = self.patch_embed(imgs)
+        gh, gw = x.shape[-2:]
+        x = x.flatten(2).transpose(1, 2)
+        x = torch.cat((self.cls_token.expand(f, -1, -1), x), dim=1) + self._pos(gh, gw)
+        x = torch.cat((x[:, :1], self.register_tokens.expand(f, -1, -1), x[:, 1:]), dim=1)
+        for blk in self.blocks:
+            x = blk(x)
+        return self.norm(x)[:, 1 + self.register_tokens.shape[1]:]
+
+
+class HeadDecoder(nn.Module):
+    def __init__(self, in_dim, out_dim, dim=1024, depth=5, num_heads=16, rope=None) -> None:
+        super().__init__()
+        self.project = nn.Linear(in_dim, dim)
+        self.blocks = nn.ModuleList([Block(dim, num_heads, DenseAttentionRope, rope=rope) for _ in range(depth)])
+        self.linear_out = nn.Linear(dim, out_dim)
+
+    def forward(self, x: Tensor, xpos: Tensor) -> Tensor:
+        x = self.project(x)
+        for blk in self.blocks:
+            x = blk(x, xpos=xpos)
+        return self.linear_out(x)
+
+
+class PixelShuffleHead(nn.Module):
+    def __init__(self, patch: int, dim: int, out_dim: int) -> None:
+        super().__init__()
+        self.patch = patch
+        self.proj = nn.Linear(dim, out_dim * patch * patch)
+
+    def forward(self, tokens: Tensor, gh: int, gw: int) -> Tensor:  # [F, gh*gw, dim] -> [F, H, W, out]
+        f = tokens.shape[0]
+        feat = self.proj(tokens).transpose(-1, -2).reshape(f, -1, gh, gw)
+        return F.pixel_shuffle(feat, self.patch).permute(0, 2, 3, 1)
+
+
+class PoseHead(nn.Module):
+    """Frame tokens -> 4x4 camera-to-world matrix (rotation from two 3-vectors by Gram-Schmidt, translation)."""
+
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.mlp = nn.Sequential(nn.Linear(dim, dim), nn.GELU(), nn.Linear(dim, 9))
+
+    def forward(self, tokens: Tensor) -> Tensor:  # [F, T, dim] -> [F, 4, 4]
+        p = self.mlp(tokens.mean(dim=1)).float()
+        a, b, t = p[:, 0:3], p[:, 3:6], p[:, 6:9]
+        e1 = F.normalize(a + torch.tensor([1.0, 0.0, 0.0], device=p.device), dim=-1)
+        b = b + torch.tensor([0.0, 1.0, 0.0], device=p.device)
+        e2 = F.normalize(b - (e1 * b).sum(-1, keepdim=True) * e1, dim=-1)
+        e3 = torch.cross(e1, e2, dim=-1)
+        pose = torch.zeros((p.shape[0], 4, 4), device=p.device)
+        pose[:, :3, :3] = torch.stack((e1, e2, e3), dim=-1)
+        pose[:, :3, 3] = t
+        pose[:, 3, 3] = 1.0
+        return pose
+
+
+class Pi3SparseLike(nn.Module):
+    def __init__(self, dim=1024, enc_depth=24, dec_depth=36, num_heads=16, head_depth=5, patch=14, grid=(37, 28),
+                 num_register=5, block_tokens=64, topk=16, rope_freq=100.0) -> None:
+        super().__init__()
+        assert dec_depth % 2 == 0 and int(block_tokens ** 0.5) ** 2 == block_tokens
+        self.patch = patch
+        self.encoder = PatchEncoder(dim, enc_depth, num_heads, patch, grid)
+        self.rope = RoPE2D(freq=rope_freq, max_positions=max(grid) + 2)
+        self.register_token = nn.Parameter(torch.randn(1, num_register, dim) * 1e-6)
+        self.local_decoder = nn.ModuleList([
+            Block(dim, num_heads, DenseAttentionRope, init_values=0.01, qk_norm=True, rope=self.rope)
+            for _ in range(dec_depth // 2)])
+        self.global_decoder = nn.ModuleList([
+            Block(dim, num_heads, SparseFlashAttentionRope, init_values=0.01, qk_norm=True, rope=self.rope,
+                  block_size=int(block_tokens ** 0.5), topk=topk)
+            for _ in range(dec_depth // 2)])
+        self.point_decoder = HeadDecoder(2 * dim, dim, dim, head_depth, num_heads, self.rope)
+        self.conf_decoder = HeadDecoder(2 * dim, dim, dim, head_depth, num_heads, self.rope)
+        self.camera_decoder = HeadDecoder(2 * dim, dim // 2, dim, head_depth, num_heads, self.rope)
+        self.point_head = PixelShuffleHead(patch, dim, 3)
+        self.conf_head = PixelShuffleHead(patch, dim, 1)
+        self.camera_head = PoseHead(dim // 2)
+        self.register_buffer("image_mean", torch.tensor([0.485, 0.456, 0.406]).view(1, 3, 1, 1))
+        self.register_buffer("image_std", torch.tensor([0.229, 0.224, 0.225]).view(1, 3, 1, 1))
+
+    def _positions(self, f: int, gh: int, gw: int, device) -> Tensor:
+        yy, xx = torch.meshgrid(torch.arange(gh, device=device), torch.arange(gw, device=device), indexing="ij")
+        patch = torch.stack((yy, xx), dim=-1).reshape(gh * gw, 2) + 1           # register tokens sit at (0, 0)
+        reg = torch.zeros((self.register_token.shape[1], 2), dtype=patch.dtype, device=device)
+        return torch.cat((reg, patch), dim=0)[None].expand(f, -1, -1).contiguous()
+
+    def forward(self, imgs: Tensor) -> dict:
+        """imgs [B, F, 3, H, W] in [0,1] -> dict(points, local_points, conf, camera_poses)."""
+        b, f, _, hh, ww = imgs.shape
+        gh, gw = hh // self.patch, ww // self.patch
+        x = ((imgs - self.image_mean) / self.image_std).reshape(b * f, 3, hh, ww).to(self.register_token.dtype)
+        x = self.encoder(x)                                                        # [B*F, gh*gw, dim]
+        x = torch.cat((self.register_token.expand(b * f, -1, -1), x), dim=1)       # [B*F, T, dim]
+        t = x.shape[1]
+        pos = self._positions(b * f, gh, gw, x.device)                             # [B*F, T, 2]
+        local_out = None
+        for local_blk, global_blk in zip(self.local_decoder, self.global_decoder):
+            x = local_blk(x, xpos=pos)
+            local_out = x
+            x = global_blk(x.reshape(b, f * t, -1), xpos=pos.reshape(b, f * t, 2)).reshape(b * f, t, -1)
+        feat = torch.cat((local_out, x), dim=-1)
+        nreg = self.register_token.shape[1]
+        pts = self.point_head(self.point_decoder(feat, pos)[:, nreg:], gh, gw).float()
+        conf = self.conf_head(self.conf_decoder(feat, pos)[:, nreg:], gh, gw).float()
+        poses = self.camera_head(self.camera_decoder(feat, pos)).reshape(b, f, 4, 4)
+        xy, z = pts.split([2, 1], dim=-1)
+        z = torch.exp(z)
+        local_points = torch.cat((xy * z, z), dim=-1).reshape(b, f, gh * self.patch, gw * self.patch, 3)
+        homog = torch.cat((local_points, torch.ones_like(local_points[..., :1])), dim=-1)
+        points = torch.einsum("bnij,bnhwj->bnhwi", poses, homog)[..., :3]
+        return dict(points=points, local_points=local_points,
+                    conf=conf.reshape(b, f, gh * self.patch, gw * self.patch, 1), camera_poses=poses)
