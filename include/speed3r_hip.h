@@ -64,7 +64,10 @@ int s3r_pool_mean(const void* x, void* y, int B, int H, int64_t N, int D, int bl
  *   scores[b,h,i,j] = raw fp32 q[i].k[j]                      (optional, [B,H,Lq,Lk] contiguous)
  * When `scores` is given the indices are computed from exactly those stored values, so
  * s3r_topk_rows() on `scores` reproduces `topk_idx` bit for bit.  When `scores` is NULL the
- * selection is fused into the attention kernel and the scores never reach HBM.
+ * scores never reach HBM: the attention output comes from a dense sweep of the selection
+ * kernel and the indices from a top-k-only kernel that recomputes the scores on chip
+ * (bf16/fp16, D == 64, K in {1,2,4,8,16,32}; two launches on `stream`).  `o` may be NULL when
+ * only the indices are wanted (MFMA path), `topk_idx` may be NULL when only the attention is.
  * Requires D <= 64 (D == 64 for the MFMA path), K a power of two <= 64.
  */
 int s3r_compressed_attn_topk(const void* q, const void* k, const void* v,

@@ -33,7 +33,7 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
                                         int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
                                         int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t som,
                                         float softmax_scale, int dtype, void* stream) {
-  if (!q || !k || !v || !o) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: null pointer");
+  if (!q || !k || !v || (!o && !topk_idx)) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: null pointer");
   if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || D <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: non-positive size");
   if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: dtype %d", dtype);
   if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: head_dim %d > 64", D);
@@ -55,6 +55,7 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
     return fail(S3R_ERR_UNSUPPORTED,
                 "s3r_compressed_attn_topk: fused selection needs bf16/fp16, head_dim 64, 16-byte aligned tensors; "
                 "pass a scores buffer for other shapes");
+  if (!o) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: indices without the attention output need the MFMA path");
   int rc = launch_attn_simple(p, dtype, /*select=*/false, stream);
   if (rc != S3R_OK) return rc;
   if (topk_idx != nullptr) rc = s3r_topk_rows(scores, topk_idx, (int64_t)B * H * Lq, Lk, Lk, K, stream);

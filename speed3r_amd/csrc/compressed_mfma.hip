@@ -25,6 +25,7 @@
 #include "s3r_common.h"
 #include "attn_params.h"
 #include <type_traits>
+#include <type_traits>
 #include <utility>
 
 namespace s3r {
@@ -106,13 +107,13 @@ constexpr int kTile = 64 * 64;  // elements per LDS tile
 constexpr int kQSlots = 16;     // LDS queue slots per lane: kQSlots-1 entries and one dump slot for non-survivors
 constexpr int kQCap = kQSlots;  // width of the merge network (entry kQSlots-1 is always empty)
 
-template <typename E, int KTOP /* 0: no fused selection */>
-__global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
+template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */>
+__global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compressed_mfma_kernel(AttnParams p) {
   typedef typename Mma<E>::V8 V8;
   constexpr bool FUSED = KTOP > 0;
   constexpr int KL = FUSED ? KTOP : 1;  // list length per lane
   __shared__ __attribute__((aligned(1024))) E Ks[2][kTile];
-  __shared__ __attribute__((aligned(1024))) E Vs[2][kTile];
+  __shared__ __attribute__((aligned(1024))) E Vs[FUSED ? 1 : 2][FUSED ? 8 : kTile];  // the top-k-only kernel stages K tiles alone
   __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][FUSED ? kQSlots : 1][64];
   __shared__ __attribute__((aligned(16))) float sstage[FUSED ? 1 : 4][FUSED ? 4 : 32 * 64];  // score-store staging (unfused launches)
 
@@ -170,17 +171,21 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
       *reinterpret_cast<uint4*>(&Vs[buf][r * 64 + ld_pos * 8]) = vr[i];
     }
   };
-  // second pass of the fused selection: K tiles only, two per step (the second one of a pair lives in the V buffer)
-  auto fetch_kk = [&](int64_t start) {
+  // top-k-only sweeps: K tiles alone
+  auto fetch_k = [&](int64_t start) {
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const int r = ld_row + 32 * i;
       int64_t row = start + r;
       row = row < Lk ? row : Lk - 1;
       kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
-      row = start + 64 + r;
-      row = row < Lk ? row : Lk - 1;
-      vr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
+    }
+  };
+  auto stash_k = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int r = ld_row + 32 * i;
+      *reinterpret_cast<uint4*>(&Ks[buf][r * 64 + ld_pos * 8]) = kr[i];
     }
   };
   // per-lane LDS read offsets (bytes)
@@ -236,6 +241,7 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
   const int gsz = (ntiles + 127) / 128;
   uint16_t* gmax = FUSED ? reinterpret_cast<uint16_t*>(&queue[wave][0][0]) : nullptr;
   float gm = -INFINITY;
+  if constexpr (!FUSED) {
   fetch(0);
   stash(0);
   if (ntiles > 1) fetch(64);
@@ -309,15 +315,6 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
     mx = xh_max(mx);
-    if constexpr (FUSED) {
-      gm = fmaxf(gm, mx);
-      if ((t + 1) % gsz == 0 || t + 1 == ntiles) {
-        const uint32_t u = __float_as_uint(gm);
-        const uint32_t down = (u >> 16) + (((u >> 31) != 0 && (u & 0xffffu) != 0) ? 1u : 0u);  // negative: one step further down
-        if (hh == 0) gmax[(t / gsz) * 32 + c] = (uint16_t)down;
-        gm = -INFINITY;
-      }
-    }
     const float m_new = fmaxf(m_i, mx * sl2);
     const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
     float rowsum = 0.f;
@@ -373,8 +370,78 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
     if (p.lse != nullptr && hh == 0)
       p.lse[((int64_t)b * p.H + h) * Lq + qrow] = l > 0.f ? (m_i + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
   }
+  }  // !FUSED
 
   if constexpr (FUSED) {
+    // One sweep over the key tiles (K tiles double-buffered in LDS, 48 KB per workgroup in all: three workgroups per
+    // compute unit): S^T by MFMA, then either the group maxima (first sweep) or the candidate filter (second sweep).
+    auto sweep = [&](auto filter_tag) {
+      constexpr bool FILTER = decltype(filter_tag)::value;
+      fetch_k(0);
+      stash_k(0);
+      if (ntiles > 1) fetch_k(64);
+      for (int t = 0; t < ntiles; t++) {
+        const int buf = t & 1;
+        __syncthreads();
+        if (t + 1 < ntiles) stash_k(buf ^ 1);
+        if (t + 2 < ntiles) fetch_k((int64_t)(t + 2) * 64);
+        {
+          const int64_t start = (int64_t)t * 64;
+          const bool partial = start + 64 > Lk;
+          f32x16 st[2];
+          const char* kbase = reinterpret_cast<const char*>(&Ks[buf][0]);
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+              Frag f;
+              f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
+              st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
+            }
+          }
+          const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
+          if constexpr (!FILTER) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) {
+                const bool valid = !partial || (kt * 32 + 8 * (r >> 2) + (r & 3) < lim);
+                mx = fmaxf(mx, valid ? st[kt][r] : -INFINITY);
+              }
+            gm = fmaxf(gm, xh_max(mx));
+            if ((t + 1) % gsz == 0 || t + 1 == ntiles) {
+              const uint32_t u = __float_as_uint(gm);
+              const uint32_t down = (u >> 16) + (((u >> 31) != 0 && (u & 0xffffu) != 0) ? 1u : 0u);  // negative: one step further down
+              if (hh == 0) gmax[(t / gsz) * 32 + c] = (uint16_t)down;
+              gm = -INFINITY;
+            }
+          } else {
+            const uint32_t col0 = (uint32_t)start + 4 * hh;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
+#pragma unroll
+              for (int e8 = 0; e8 < 8; e8++) {
+                const int kt = g >> 1, r = (g & 1) * 8 + e8;
+                const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
+                const float s = st[kt][r];
+                bool pass = !(s < thr);
+                if (partial) pass = pass && (koff < lim);
+                // no branch: every lane writes, non-survivors into the dump slot
+                uint2* dst = qlane + (pass ? qn : kQSlots - 1) * 64;
+                *dst = make_uint2(__float_as_uint(s), col0 + koff);
+                qn += pass ? 1 : 0;
+              }
+              if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
+            }
+          }
+        }
+      }
+    };
+    // First sweep: the maximum raw score of every group of gsz key tiles, per query row.
+    sweep(std::false_type{});
     // Threshold: the K-th largest group maximum of the row.  K different scores (one per group) are at least that
     // large, so a score below it is not among the K largest, whatever the tie-break.  With fewer than K groups
     // the threshold stays -inf and every score is a candidate.
@@ -395,56 +462,10 @@ __global__ __launch_bounds__(256, 2) void compressed_mfma_kernel(AttnParams p) {
       thr0 = qvalid ? top[KL - 1] : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
       thr = thr0;
     }
-    // Second pass: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
+    // Second sweep: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
     // through the lane's queue into its exact list.
-    __syncthreads();  // every wave is done with the tile buffers of the first pass (and with its own group maxima)
-    const int npairs = (ntiles + 1) / 2;
-    fetch_kk(0);
-    stash(0);
-    if (npairs > 1) fetch_kk(128);
-    for (int tp = 0; tp < npairs; tp++) {
-      const int buf = tp & 1;
-      __syncthreads();
-      if (tp + 1 < npairs) stash(buf ^ 1);
-      if (tp + 2 < npairs) fetch_kk((int64_t)(tp + 2) * 128);
-#pragma unroll
-      for (int half = 0; half < 2; half++) {
-        const int64_t start = (int64_t)tp * 128 + half * 64;
-        if (start >= Lk) break;  // odd number of tiles
-        const bool partial = start + 64 > Lk;
-        f32x16 st[2];
-        const char* kbase = reinterpret_cast<const char*>(half == 0 ? &Ks[buf][0] : &Vs[buf][0]);
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++) {
-#pragma unroll
-          for (int r = 0; r < 16; r++) st[kt][r] = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < 4; ks++) {
-            Frag f;
-            f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
-            st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
-          }
-        }
-        const int lim = (int)(Lk - start) - 4 * hh;
-        const uint32_t col0 = (uint32_t)start + 4 * hh;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
-#pragma unroll
-          for (int e8 = 0; e8 < 8; e8++) {
-            const int kt = g >> 1, r = (g & 1) * 8 + e8;
-            const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
-            const float s = st[kt][r];
-            bool pass = !(s < thr);
-            if (partial) pass = pass && (koff < lim);
-            // no branch: every lane writes, non-survivors into the dump slot
-            uint2* dst = qlane + (pass ? qn : kQSlots - 1) * 64;
-            *dst = make_uint2(__float_as_uint(s), col0 + koff);
-            qn += pass ? 1 : 0;
-          }
-          if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
-        }
-      }
-    }
+    __syncthreads();  // every wave is done with the tile buffers of the first sweep
+    sweep(std::true_type{});
     drain();
     // the partner lane's list, then the K best of both, descending
     uint64_t other[KL];
@@ -490,16 +511,37 @@ bool compressed_fused_topk_available(int K) { return K == 1 || K == 2 || K == 4 
 
 int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream) {
   hipStream_t st = (hipStream_t)stream;
-  // fused selection when indices are wanted and no score buffer is given; with a score buffer the indices come
-  // from exactly the stored values through the row-wise kernel
-  const bool fused = p.topk_idx != nullptr && p.scores == nullptr;
-  if (fused && !compressed_fused_topk_available(p.K))
+  // With a score buffer: one kernel writes the attention output and the raw scores, the row-wise kernel selects
+  // from exactly those values.  Without one: the attention runs as a dense sweep of the selection kernel (its
+  // pipelined loop is the fastest attention loop of this library) and the indices come from the top-k-only kernel
+  // (two sweeps over S, scores never leave the chip).
+  if (p.scores != nullptr) {
+    int rc = dtype == S3R_BF16 ? cmp::launch_e<bf16_t>(p, false, st) : cmp::launch_e<f16_t>(p, false, st);
+    if (rc != S3R_OK) return rc;
+    if (p.topk_idx != nullptr)
+      rc = s3r_topk_rows(p.scores, p.topk_idx, (int64_t)p.B * p.H * p.Lq, (int)p.Lk, p.Lk, p.K, stream);
+    return rc;
+  }
+  if (p.topk_idx != nullptr && !compressed_fused_topk_available(p.K))
     return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}; pass a scores buffer");
-  int rc = dtype == S3R_BF16 ? cmp::launch_e<bf16_t>(p, fused, st) : cmp::launch_e<f16_t>(p, fused, st);
-  if (rc != S3R_OK) return rc;
-  if (p.topk_idx != nullptr && !fused)
-    rc = s3r_topk_rows(p.scores, p.topk_idx, (int64_t)p.B * p.H * p.Lq, (int)p.Lk, p.Lk, p.K, stream);
-  return rc;
+  if (p.o != nullptr) {
+    int rc;
+    if (p.Lq == p.Lk && p.skn < (1 << 20) && p.svn < (1 << 20)) {
+      AttnParams d = p;
+      d.idx = nullptr;  // dense sweep
+      d.topk_idx = nullptr;
+      d.block = 64;
+      d.merge_out = nullptr;
+      rc = launch_select_pipe(d, dtype, stream);
+    } else {
+      AttnParams a = p;
+      a.topk_idx = nullptr;
+      rc = dtype == S3R_BF16 ? cmp::launch_e<bf16_t>(a, false, st) : cmp::launch_e<f16_t>(a, false, st);
+    }
+    if (rc != S3R_OK) return rc;
+  }
+  if (p.topk_idx != nullptr) return dtype == S3R_BF16 ? cmp::launch_e<bf16_t>(p, true, st) : cmp::launch_e<f16_t>(p, true, st);
+  return S3R_OK;
 }
 
 }  // namespace s3r

@@ -31,7 +31,9 @@ using namespace sel;
 
 constexpr int kHalf = 32 * 64;  // elements per half tile
 
-template <typename E>
+// DENSE: no index list, every query block attends to all key tiles in order (the compressed branch's attention over
+// the pooled tokens runs through this instance).
+template <typename E, bool DENSE>
 __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
   const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
   E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
-  const int32_t* idx_row = p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
+  const int32_t* idx_row = DENSE ? nullptr : p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
 
   auto k_half = [&](auto hf) -> E* {
     if constexpr (decltype(hf)::value == 0) return reinterpret_cast<E*>(lds_k0) + wave * kHalf;
@@ -76,12 +78,22 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   typedef std::integral_constant<int, 1> H1;
 
   // index list: full tiles go through the pipeline, occurrences of the ragged last block come after it
-  const int32_t my_idx = lane < p.K ? idx_row[lane] : -1;
+  int32_t my_idx = -1;
   const int32_t ragged_blk = (N & 63) ? (int32_t)(N >> 6) : -1;
-  const bool my_valid = my_idx >= 0 && (int64_t)my_idx * 64 < N;
-  uint64_t todo = __ballot(my_valid && my_idx != ragged_blk);
-  int n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
-  const int n_full = __popcll(todo);
+  bool my_valid = false;
+  uint64_t todo = 0;
+  int n_ragged, n_full;
+  int dense_next = 0;  // DENSE: the next tile of the sweep
+  if constexpr (DENSE) {
+    n_full = (int)(N >> 6);
+    n_ragged = (N & 63) ? 1 : 0;
+  } else {
+    my_idx = lane < p.K ? idx_row[lane] : -1;
+    my_valid = my_idx >= 0 && (int64_t)my_idx * 64 < N;
+    todo = __ballot(my_valid && my_idx != ragged_blk);
+    n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
+    n_full = __popcll(todo);
+  }
   if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
@@ -367,6 +379,11 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   if (n_full > 0) {
     int64_t last_start = 0;
     auto pop_or_last = [&]() -> int64_t {  // branch-free: next full tile, or the last one again
+      if constexpr (DENSE) {
+        last_start = (int64_t)(dense_next < n_full ? dense_next : n_full - 1) * 64;
+        dense_next++;
+        return last_start;
+      }
       const bool any = todo != 0;
       const int t = any ? __ffsll((unsigned long long)todo) - 1 : 0;
       const int64_t s = (int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64;
@@ -417,11 +434,15 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
 
   if (redo) {  // rare: recompute the query block with the online softmax
     reset_state();
-    uint64_t again = __ballot(my_valid && my_idx != ragged_blk);
-    while (again) {
-      const int t = __ffsll((unsigned long long)again) - 1;
-      again &= again - 1;
-      robust_tile((int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64);
+    if constexpr (DENSE) {
+      for (int t = 0; t < n_full; t++) robust_tile((int64_t)t * 64);
+    } else {
+      uint64_t again = __ballot(my_valid && my_idx != ragged_blk);
+      while (again) {
+        const int t = __ffsll((unsigned long long)again) - 1;
+        again &= again - 1;
+        robust_tile((int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64);
+      }
     }
   }
   for (; n_ragged > 0; n_ragged--) robust_tile((int64_t)ragged_blk * 64);
@@ -493,10 +514,15 @@ int launch_select_pipe(const AttnParams& p, int dtype, void* stream) {
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)total), blk(256);
-  if (dtype == S3R_BF16)
-    hipLaunchKernelGGL(pipe::select_pipe_kernel<bf16_t>, grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
-  else
-    hipLaunchKernelGGL(pipe::select_pipe_kernel<f16_t>, grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
+  const bool dense = p.idx == nullptr;  // no index list: every query block sweeps all key tiles
+  if (dense && p.Lq != p.Lk) return fail(S3R_ERR_UNSUPPORTED, "dense sweep: Lq %lld != Lk %lld", (long long)p.Lq, (long long)p.Lk);
+  if (dtype == S3R_BF16) {
+    if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<bf16_t, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
+    else hipLaunchKernelGGL((pipe::select_pipe_kernel<bf16_t, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
+  } else {
+    if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<f16_t, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
+    else hipLaunchKernelGGL((pipe::select_pipe_kernel<f16_t, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
+  }
   return check_launch("select_pipe_kernel");
 }
 

@@ -140,7 +140,9 @@ def test_fused_selection_equals_selection_from_stored_scores(dtype, k, lq, lk):
     want = oracle.topk_from_scores(scores.cpu(), k)
     np.testing.assert_array_equal(idx_m.cpu().numpy(), want)
     np.testing.assert_array_equal(idx_f.cpu().numpy(), want)
-    assert torch.equal(o_f, o_m)
+    # the two routes compute the attention output with different kernels (dense sweep of the selection kernel vs the
+    # score-writing kernel): same mathematics, different summation order
+    assert max_abs(o_f, o_m.float()) <= 2e-2
 
 
 def test_fused_selection_special_scores():
