@@ -41,8 +41,10 @@ template <> struct Mma<f16_t> {
   static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
 };
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 union Frag {
   uint4 u;
+  u32x4 w;
   bf16x8 b;
   f16x8 h;
   s16x4 s[2];
@@ -104,17 +106,41 @@ template <int N> __device__ __forceinline__ void merge_top_desc(uint64_t (&a)[N]
 }
 
 constexpr int kTile = 64 * 64;  // elements per LDS tile
-constexpr int kQSlots = 16;     // LDS queue slots per lane: kQSlots-1 entries and one dump slot for non-survivors
-constexpr int kQCap = kQSlots;  // width of the merge network (entry kQSlots-1 is always empty)
+constexpr int kQCap = 16;       // width of the merge network that folds a lane's queue into its list
+// Top-k-only kernel, per list length: LDS queue slots per lane (the last one is the dump slot of non-survivors) and
+// K tiles in the LDS ring.  Up to 16: 28 KB of queues + 24 KB of tiles, three workgroups per compute unit;
+// above: 32 KB + 48 KB, two.
+template <int KTOP> struct TopkCfg {
+  static constexpr int kQSlots = KTOP <= 16 ? 14 : 16;
+  static constexpr int kRing = KTOP <= 16 ? 3 : 6;
+};
+template <> struct TopkCfg<0> {
+  static constexpr int kQSlots = 1;
+  static constexpr int kRing = 2;
+};
+
+// LDS read whose completion the caller waits for itself (lds_reads_done): the compiler neither knows that it reads
+// LDS nor when it lands, so it adds no wait for transfers into other LDS buffers that are still in flight.
+template <int OFF> __device__ __forceinline__ u32x4 lds_read16_async(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+__device__ __forceinline__ void lds_reads_done(u32x4 (&a)[2][4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]), "+v"(a[1][0]), "+v"(a[1][1]), "+v"(a[1][2]), "+v"(a[1][3]));
+}
 
 template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */>
 __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compressed_mfma_kernel(AttnParams p) {
   typedef typename Mma<E>::V8 V8;
   constexpr bool FUSED = KTOP > 0;
   constexpr int KL = FUSED ? KTOP : 1;  // list length per lane
-  __shared__ __attribute__((aligned(1024))) E Ks[2][kTile];
+  constexpr int kQSlots = TopkCfg<KTOP>::kQSlots;
+  constexpr int NB = TopkCfg<KTOP>::kRing;
+  __shared__ __attribute__((aligned(1024))) E Ks[NB][kTile];
   __shared__ __attribute__((aligned(1024))) E Vs[FUSED ? 1 : 2][FUSED ? 8 : kTile];  // the top-k-only kernel stages K tiles alone
-  __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][FUSED ? kQSlots : 1][64];
+  __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][kQSlots][64];
   __shared__ __attribute__((aligned(16))) float sstage[FUSED ? 1 : 4][FUSED ? 4 : 32 * 64];  // score-store staging (unfused launches)
 
   const int tid = threadIdx.x;
@@ -171,23 +197,6 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
       *reinterpret_cast<uint4*>(&Vs[buf][r * 64 + ld_pos * 8]) = vr[i];
     }
   };
-  // top-k-only sweeps: K tiles alone
-  auto fetch_k = [&](int64_t start) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const int r = ld_row + 32 * i;
-      int64_t row = start + r;
-      row = row < Lk ? row : Lk - 1;
-      kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
-    }
-  };
-  auto stash_k = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const int r = ld_row + 32 * i;
-      *reinterpret_cast<uint4*>(&Ks[buf][r * 64 + ld_pos * 8]) = kr[i];
-    }
-  };
   // per-lane LDS read offsets (bytes)
   const int i16 = lane & 15;
   const int tr_row = 4 * hh + (i16 >> 2);
@@ -198,8 +207,8 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
   uint64_t list[KL];  // descending
 #pragma unroll
   for (int i = 0; i < KL; i++) list[i] = 0;
-  float thr = __uint_as_float(0xFFFFFFFFu);  // a NaN: "s < thr" is false for every s, so everything passes
-  float thr0 = -INFINITY;                    // the row's threshold from the group maxima; thr never drops below it
+  float thr = -INFINITY;   // survivors are the scores >= thr
+  float thr0 = -INFINITY;  // the row's threshold from the group maxima; thr never drops below it
   int qn = 0;
   uint2* qlane = FUSED ? &queue[wave][0][lane] : nullptr;  // entry e at qlane[e * 64]
   const uint32_t lkm1 = (uint32_t)(Lk - 1);
@@ -208,9 +217,12 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
     uint64_t cand[kQCap];
 #pragma unroll
     for (int e = 0; e < kQCap; e++) {
-      const uint2 v = qlane[e * 64];
-      const uint64_t key = ((uint64_t)sortable_key(__uint_as_float(v.x)) << 32) | (uint64_t)(lkm1 - v.y);
-      cand[e] = e < qn ? key : 0;
+      cand[e] = 0;
+      if (e < kQSlots - 1) {
+        const uint2 v = qlane[e * 64];
+        const uint64_t key = ((uint64_t)sortable_key(__uint_as_float(v.x)) << 32) | (uint64_t)(lkm1 - v.y);
+        cand[e] = e < qn ? key : 0;
+      }
     }
     bitonic_sort_desc<kQCap>(cand);
     if constexpr (KL == kQCap) {
@@ -229,16 +241,17 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
       merge_top_desc<KL>(list, wide);
     }
     qn = 0;
-    // threshold = score of the list's last entry (key 0, a filler, maps to a NaN: everything passes)
+    // threshold = score of the list's last entry (key 0, a filler, maps to a NaN, which fmaxf drops: thr0 remains)
     const uint32_t k32 = (uint32_t)(list[KL - 1] >> 32);
     thr = fmaxf(__uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)), thr0);  // fmaxf drops the NaN
   };
 
   const int ntiles = (int)((Lk + 63) / 64);
-  // Fused selection, first pass: the maxima of the raw scores over groups of gsz key tiles (at most 128 groups per
-  // row) go to the wave's queue memory, which is idle until the second pass: gmax[group * 32 + row], as 16-bit
+  // Fused selection, first pass: the maxima of the raw scores over groups of gsz key tiles (at most kGroups groups
+  // per row) go to the wave's queue memory, which is idle until the second pass: gmax[group * 32 + row], as 16-bit
   // floats (the upper half of the fp32 pattern) rounded DOWN, so that a threshold taken from them is still a lower bound.
-  const int gsz = (ntiles + 127) / 128;
+  constexpr int kGroups = kQSlots * 8;  // 64 bytes per group in kQSlots * 512 bytes of queue
+  const int gsz = (ntiles + kGroups - 1) / kGroups;
   uint16_t* gmax = FUSED ? reinterpret_cast<uint16_t*>(&queue[wave][0][0]) : nullptr;
   float gm = -INFINITY;
   if constexpr (!FUSED) {
@@ -373,23 +386,50 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
   }  // !FUSED
 
   if constexpr (FUSED) {
-    // One sweep over the key tiles (K tiles double-buffered in LDS, 48 KB per workgroup in all: three workgroups per
-    // compute unit): S^T by MFMA, then either the group maxima (first sweep) or the candidate filter (second sweep).
+    // One sweep over the key tiles: S^T by MFMA, then either the group maxima (first sweep) or the candidate filter
+    // (second sweep).  K tiles go global -> LDS by direct transfers into a ring of NB buffers, NB - 1 tiles ahead of
+    // the tile being read; wave w moves rows 16w .. 16w+15 of a tile (two instructions of 8 rows).  LDS chunk
+    // (row, c') holds head_dim chunk c' ^ (row & 7).  Rows beyond Lk re-read the last row (they are masked).
+    const uint32_t krow_bytes = (uint32_t)p.skn * (uint32_t)sizeof(E);
+    const int dl_row = wave * 16 + (lane >> 3);
+    const uint32_t dl_chunk = (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
+    auto dma_tile = [&](int t, int buf) {  // tiles past the end repeat the last one (never read)
+      const int tt = t < ntiles ? t : ntiles - 1;
+      const int64_t start = (int64_t)tt * 64;
+      const int rem = (int)(Lk - 1 - start);
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
+      char* dst = reinterpret_cast<char*>(&Ks[buf][0]) + wave * 2048;
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        int r = dl_row + 8 * i;
+        r = r < rem ? r : rem;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16,
+                                                 (uint32_t)r * krow_bytes + dl_chunk, 0, 0, 0);
+      }
+    };
+    const uint32_t lds_k = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(&Ks[0][0]);
+    const uint32_t kr_off = lds_k + (uint32_t)(c * 128 + ((hh ^ (c & 7)) << 4));  // A operand: lane = key row, chunk hh + 2 ks
     auto sweep = [&](auto filter_tag) {
       constexpr bool FILTER = decltype(filter_tag)::value;
-      fetch_k(0);
-      stash_k(0);
-      if (ntiles > 1) fetch_k(64);
+      for (int i = 0; i < NB - 1; i++) dma_tile(i, i);
+      int buf = 0, fill = NB - 1;  // ring positions of tile t and of tile t + NB - 1
       for (int t = 0; t < ntiles; t++) {
-        const int buf = t & 1;
-        __syncthreads();
-        if (t + 1 < ntiles) stash_k(buf ^ 1);
-        if (t + 2 < ntiles) fetch_k((int64_t)(t + 2) * 64);
+        // this wave's share of tile t has landed (transfers complete in order, two per tile, NB - 2 tiles younger) ...
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NB - 2)));
+        __builtin_amdgcn_s_barrier();  // ... and everybody's; all waves are done with tile t - 1, whose buffer is refilled now
+        dma_tile(t + NB - 1, fill);
         {
           const int64_t start = (int64_t)t * 64;
           const bool partial = start + 64 > Lk;
+          u32x4 kf[2][4];
+          const uint32_t kb = kr_off + (uint32_t)buf * (kTile * (uint32_t)sizeof(E));
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) {
+            kf[0][ks] = lds_read16_async<0>(kb ^ (ks << 5));
+            kf[1][ks] = lds_read16_async<32 * 128>(kb ^ (ks << 5));
+          }
+          lds_reads_done(kf);
           f32x16 st[2];
-          const char* kbase = reinterpret_cast<const char*>(&Ks[buf][0]);
 #pragma unroll
           for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
@@ -397,20 +437,26 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
               Frag f;
-              f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
+              f.w = kf[kt][ks];
               st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
             }
           }
-          const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
-          if constexpr (!FILTER) {
-            float mx = -INFINITY;
+          buf = buf + 1 == NB ? 0 : buf + 1;
+          fill = fill + 1 == NB ? 0 : fill + 1;
+          if (partial) {  // last tile only: keys beyond Lk get a score that neither raises a maximum nor passes the filter
+            const int lim = (int)(Lk - start) - 4 * hh;  // register r of tile kt holds key kt*32 + 4hh + 8(r/4) + r%4
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-              for (int r = 0; r < 16; r++) {
-                const bool valid = !partial || (kt * 32 + 8 * (r >> 2) + (r & 3) < lim);
-                mx = fmaxf(mx, valid ? st[kt][r] : -INFINITY);
-              }
+              for (int r = 0; r < 16; r++)
+                if (kt * 32 + 8 * (r >> 2) + (r & 3) >= lim) st[kt][r] = FILTER ? __uint_as_float(0x7FC00000u) : -INFINITY;
+          }
+          if constexpr (!FILTER) {
+            float mx = st[0][0];
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
             gm = fmaxf(gm, xh_max(mx));
             if ((t + 1) % gsz == 0 || t + 1 == ntiles) {
               const uint32_t u = __float_as_uint(gm);
@@ -427,18 +473,18 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
                 const int kt = g >> 1, r = (g & 1) * 8 + e8;
                 const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
                 const float s = st[kt][r];
-                bool pass = !(s < thr);
-                if (partial) pass = pass && (koff < lim);
+                const bool pass = s >= thr;  // thr is never a NaN; a NaN score (masked key) fails
                 // no branch: every lane writes, non-survivors into the dump slot
                 uint2* dst = qlane + (pass ? qn : kQSlots - 1) * 64;
                 *dst = make_uint2(__float_as_uint(s), col0 + koff);
                 qn += pass ? 1 : 0;
               }
-              if (__any(qn > kQSlots - 1 - 8)) drain();  // at most 7 queued before a group, at most 15 after
+              if (__any(qn > kQSlots - 1 - 8)) drain();  // at most kQSlots-9 queued before a group, at most kQSlots-1 after
             }
           }
         }
       }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers issued past the last tile are done too
     };
     // First sweep: the maximum raw score of every group of gsz key tiles, per query row.
     sweep(std::false_type{});
