@@ -13,14 +13,14 @@
 // fp32, P rounded to the I/O dtype, O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16.
 //
 // Fused selection.  Every lane keeps the exact top-K of the keys IT sees (half of each tile):
-// a descending sorted list of K 64-bit keys, key = sortable(bits(score)) << 32 | (Lk-1-col),
+// a descending sorted list of K keys, key = (sortable(bits(score)), Lk-1-col) in lexicographic order,
 // in registers.  Scores are first filtered against the score of the list's last entry (one
 // compare per score; survivors are appended to a small per-lane queue in LDS).  When some
 // lane's queue is more than half full, all lanes merge their queues into their lists with a
 // register-resident bitonic network (no divergence: every lane runs the same network on its
 // own data) and refresh their thresholds.  At the end the two lanes of a query merge their
 // lists and lane < 32 writes the K indices in descending key order.  The filter is
-// conservative (anything that could enter passes), the network compares full 64-bit keys,
+// conservative (anything that could enter passes), the network compares full keys,
 // so the result is the same unique top-K as a sort of the whole row.
 #include "s3r_common.h"
 #include "attn_params.h"
@@ -66,22 +66,34 @@ __device__ __forceinline__ float xh_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// ---- register-resident bitonic networks on 64-bit keys (descending order) ----
-__device__ __forceinline__ void cex_desc(uint64_t& a, uint64_t& b) {  // a = max, b = min
-  const bool gt = a > b;
-  const uint64_t hi = gt ? a : b;
-  const uint64_t lo = gt ? b : a;
+// ---- register-resident bitonic networks (descending order) ----
+// A key is the pair (sortable bits of the score, Lk-1-col) held as ONE double, sortable * 2^21 + (Lk-1-col): exact for
+// Lk <= 2^21 (53 bits), ordered like the 64-bit integer key, and a compare-exchange is one v_max_f64 and one
+// v_min_f64 instead of a 64-bit compare and four selects.  0.0 is the filler (it decodes to column Lk-1).
+typedef double key_t;
+constexpr double kKeyScale = 2097152.0;  // 2^21
+__device__ __forceinline__ key_t make_key(uint32_t score_bits, uint32_t rev_col) {
+  return __builtin_fma((double)sortable_key(__uint_as_float(score_bits)), kKeyScale, (double)rev_col);
+}
+__device__ __forceinline__ uint32_t key_sortable(key_t k) { return (uint32_t)(k * (1.0 / kKeyScale)); }  // truncation
+__device__ __forceinline__ uint32_t key_rev_col(key_t k) {
+  const double hi = __builtin_trunc(k * (1.0 / kKeyScale));
+  return (uint32_t)__builtin_fma(hi, -kKeyScale, k);
+}
+__device__ __forceinline__ void cex_desc(key_t& a, key_t& b) {  // a = max, b = min
+  const key_t hi = __builtin_fmax(a, b);
+  const key_t lo = __builtin_fmin(a, b);
   a = hi;
   b = lo;
 }
-template <int N> __device__ __forceinline__ void bitonic_merge_desc(uint64_t (&x)[N]) {  // x bitonic -> descending
+template <int N> __device__ __forceinline__ void bitonic_merge_desc(key_t (&x)[N]) {  // x bitonic -> descending
 #pragma unroll
   for (int d = N / 2; d >= 1; d >>= 1)
 #pragma unroll
     for (int i = 0; i < N; i++)
       if ((i & d) == 0) cex_desc(x[i], x[i | d]);
 }
-template <int N> __device__ __forceinline__ void bitonic_sort_desc(uint64_t (&x)[N]) {
+template <int N> __device__ __forceinline__ void bitonic_sort_desc(key_t (&x)[N]) {
 #pragma unroll
   for (int k = 2; k <= N; k <<= 1)
 #pragma unroll
@@ -99,9 +111,9 @@ template <int N> __device__ __forceinline__ void bitonic_sort_desc(uint64_t (&x)
       }
 }
 // top-N of (descending a) U (descending b) -> a, descending
-template <int N> __device__ __forceinline__ void merge_top_desc(uint64_t (&a)[N], const uint64_t (&b)[N]) {
+template <int N> __device__ __forceinline__ void merge_top_desc(key_t (&a)[N], const key_t (&b)[N]) {
 #pragma unroll
-  for (int i = 0; i < N; i++) a[i] = a[i] > b[N - 1 - i] ? a[i] : b[N - 1 - i];  // half-cleaner: a is now bitonic
+  for (int i = 0; i < N; i++) a[i] = __builtin_fmax(a[i], b[N - 1 - i]);  // half-cleaner: a is now bitonic
   bitonic_merge_desc<N>(a);
 }
 
@@ -204,7 +216,7 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
   const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
 
   // ---- fused selection state ----
-  uint64_t list[KL];  // descending
+  key_t list[KL];  // descending
 #pragma unroll
   for (int i = 0; i < KL; i++) list[i] = 0;
   float thr = -INFINITY;   // survivors are the scores >= thr
@@ -214,35 +226,34 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
   const uint32_t lkm1 = (uint32_t)(Lk - 1);
 
   auto drain = [&]() {  // merge this lane's queue into its list; every lane runs the same network
-    uint64_t cand[kQCap];
+    key_t cand[kQCap];
 #pragma unroll
     for (int e = 0; e < kQCap; e++) {
       cand[e] = 0;
       if (e < kQSlots - 1) {
         const uint2 v = qlane[e * 64];
-        const uint64_t key = ((uint64_t)sortable_key(__uint_as_float(v.x)) << 32) | (uint64_t)(lkm1 - v.y);
-        cand[e] = e < qn ? key : 0;
+        cand[e] = e < qn ? make_key(v.x, lkm1 - v.y) : 0.0;
       }
     }
     bitonic_sort_desc<kQCap>(cand);
     if constexpr (KL == kQCap) {
       merge_top_desc<KL>(list, cand);
     } else if constexpr (KL < kQCap) {  // keep the KL best of list U cand: widen the list, merge, truncate
-      uint64_t wide[kQCap];
+      key_t wide[kQCap];
 #pragma unroll
       for (int i = 0; i < kQCap; i++) wide[i] = i < KL ? list[i] : 0;
       merge_top_desc<kQCap>(wide, cand);
 #pragma unroll
       for (int i = 0; i < KL; i++) list[i] = wide[i];
     } else {  // KL > kQCap: merge the candidates into the two (or more) halves' worth of list
-      uint64_t wide[KL];
+      key_t wide[KL];
 #pragma unroll
       for (int i = 0; i < KL; i++) wide[i] = i < kQCap ? cand[i] : 0;
       merge_top_desc<KL>(list, wide);
     }
     qn = 0;
     // threshold = score of the list's last entry (key 0, a filler, maps to a NaN, which fmaxf drops: thr0 remains)
-    const uint32_t k32 = (uint32_t)(list[KL - 1] >> 32);
+    const uint32_t k32 = key_sortable(list[KL - 1]);
     thr = fmaxf(__uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)), thr0);  // fmaxf drops the NaN
   };
 
@@ -514,18 +525,19 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
     sweep(std::true_type{});
     drain();
     // the partner lane's list, then the K best of both, descending
-    uint64_t other[KL];
+    key_t other[KL];
 #pragma unroll
     for (int i = 0; i < KL; i++) {
-      const uint32_t lo = xh_swap((uint32_t)list[i]);
-      const uint32_t hi = xh_swap((uint32_t)(list[i] >> 32));
-      other[i] = ((uint64_t)hi << 32) | lo;
+      const uint64_t bits = (uint64_t)__double_as_longlong(list[i]);
+      const uint32_t lo = xh_swap((uint32_t)bits);
+      const uint32_t hi = xh_swap((uint32_t)(bits >> 32));
+      other[i] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
     }
     merge_top_desc<KL>(list, other);
     if (qvalid && hh == 0) {
       int32_t* irow = p.topk_idx + (((int64_t)b * p.H + h) * Lq + qrow) * KL;
 #pragma unroll
-      for (int i = 0; i < KL; i++) irow[i] = (int32_t)(lkm1 - (uint32_t)list[i]);
+      for (int i = 0; i < KL; i++) irow[i] = (int32_t)(lkm1 - key_rev_col(list[i]));
     }
   }
 }
@@ -570,6 +582,8 @@ int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream) {
   }
   if (p.topk_idx != nullptr && !compressed_fused_topk_available(p.K))
     return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}; pass a scores buffer");
+  if (p.topk_idx != nullptr && (p.Lk > (1 << 21) || p.skn >= (1 << 24)))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for Lk <= 2^21 and key strides < 2^24; pass a scores buffer");
   if (p.o != nullptr) {
     int rc;
     if (p.Lq == p.Lk && p.skn < (1 << 20) && p.svn < (1 << 20)) {
