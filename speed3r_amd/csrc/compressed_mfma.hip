@@ -477,18 +477,32 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
             }
           } else {
             const uint32_t col0 = (uint32_t)start + 4 * hh;
+            const uint32_t qbase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(qlane);
 #pragma unroll
             for (int g = 0; g < 4; g++) {  // 8 scores per group, then a drain check
+              if ((g & 1) == 0) {
+                // an ordinary VALU read of the accumulator before the hand-written block below: the compiler pads
+                // the distance from the MFMA that wrote it for this instruction, not for inline assembly
+                const float settled = fmaxf(st[g >> 1][0], st[g >> 1][15]);
+                asm volatile("" ::"v"(settled));
+              }
 #pragma unroll
               for (int e8 = 0; e8 < 8; e8++) {
                 const int kt = g >> 1, r = (g & 1) * 8 + e8;
                 const int koff = kt * 32 + 8 * (r >> 2) + (r & 3);
-                const float s = st[kt][r];
-                const bool pass = s >= thr;  // thr is never a NaN; a NaN score (masked key) fails
-                // no branch: every lane writes, non-survivors into the dump slot
-                uint2* dst = qlane + (pass ? qn : kQSlots - 1) * 64;
-                *dst = make_uint2(__float_as_uint(s), col0 + koff);
-                qn += pass ? 1 : 0;
+                // Branch-free append, five VALU instructions: survivors (score >= thr; thr is never a NaN, a masked
+                // key's NaN fails) go to queue slot qn, the others to the dump slot; every lane writes (score, column).
+                uint32_t slot, col;
+                asm volatile(
+                    "v_cmp_ge_f32 vcc, %[s], %[thr]\n\t"
+                    "v_cndmask_b32 %[slot], %[dump], %[qn], vcc\n\t"
+                    "v_addc_co_u32 %[qn], vcc, 0, %[qn], vcc\n\t"
+                    "v_add_u32 %[col], %[koff], %[col0]\n\t"
+                    "v_lshl_add_u32 %[slot], %[slot], 9, %[qbase]\n\t"
+                    "ds_write2_b32 %[slot], %[s], %[col] offset1:1"
+                    : [slot] "=&v"(slot), [col] "=&v"(col), [qn] "+v"(qn)
+                    : [s] "v"(st[kt][r]), [thr] "v"(thr), [dump] "n"(kQSlots - 1), [koff] "n"(koff), [col0] "v"(col0), [qbase] "v"(qbase)
+                    : "vcc", "memory");
               }
               if (__any(qn > kQSlots - 1 - 8)) drain();  // at most kQSlots-9 queued before a group, at most kQSlots-1 after
             }
