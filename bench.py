@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
     ap.add_argument("--no-fuse-merge", action="store_true", help="run selection attention and the gated merge as two kernels")
+    ap.add_argument("--overlap", action="store_true",
+                    help="run the index kernel on a second stream beside the pooling of v and the compressed attention")
     ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "copy"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
@@ -148,27 +150,11 @@ def main() -> int:
     mat = True if args.materialize_scores else None
 
     fused = not args.no_fuse_merge
-    names = ["pool", "compressed_topk", "select_merge"] if fused else ["pool", "compressed_topk", "select", "merge"]
+    overlap = args.overlap and not args.materialize_scores
 
-    def step(events=None):
-        def mark(i):
-            if events is not None:
-                events[i].record()
-        mark(0)
-        qc, kc, vc = s3r.pool_mean(qd, block), s3r.pool_mean(kd, block), s3r.pool_mean(vd, block)
-        mark(1)
-        o_cmp, idx = s3r.compressed_attn_topk(qc, kc, vc, topk, materialize_scores=mat)
-        mark(2)
-        if fused:   # the merge runs in the selection kernel's epilogue (same bits as the two kernels)
-            out = s3r.select_attn_merge(qd, kd, vd, idx, o_cmp, gd, block)
-            assert out is not None, "the library has no fused selection+merge kernel for this shape"
-            mark(3)
-            return out
-        o_sel = s3r.select_attn(qd, kd, vd, idx, block)
-        mark(3)
-        out = s3r.gated_merge(o_cmp, o_sel, gd, block)
-        mark(4)
-        return out
+    def step(timeline=None):
+        return s3r.sparse_global_attention(qd, kd, vd, gd, block, topk, materialize_scores=mat, fuse_merge=fused,
+                                           overlap=overlap, timeline=timeline)
 
     if args.only:
         with torch.no_grad():
@@ -196,7 +182,7 @@ def main() -> int:
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
-        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+        evs = [{} for _ in range(args.steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(args.steps):
@@ -207,10 +193,21 @@ def main() -> int:
 
     ms_per_step = wall * 1e3 / args.steps
     nc = -(-n // block)
-    kern_ms = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
+    def span(a, b):
+        return sum(e[a].elapsed_time(e[b]) for e in evs) / args.steps
+
+    sel_name = "select_merge" if fused else "select"
+    if overlap:   # the index kernel runs on a second stream beside the pooling of v and the compressed attention
+        kern_ms = {"pool+compressed_topk (two streams)": span("start", "select")}
+    else:
+        kern_ms = {"pool": span("start", "pooled"), "compressed_topk": span("pooled", "select")}
+    if fused:
+        kern_ms["select_merge"] = span("select", "end")
+    else:
+        kern_ms["select"] = span("select", "merge")
+        kern_ms["merge"] = span("merge", "end")
     f_sel = workloads.selection_flops(n, topk)
     f_cmp = workloads.compressed_flops(n)
-    sel_name = "select_merge" if fused else "select"
     sel_tflops = f_sel / (kern_ms[sel_name] * 1e-3) / 1e12
     es = 2 if cfg.dtype != torch.float32 else 4
     pool_bytes = 3 * (n + nc) * 16 * 64 * es
@@ -237,7 +234,7 @@ def main() -> int:
         },
         "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
         "kernels_ms": kern_ms,
-        "hbm_gbs": {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9,
+        "hbm_gbs": {**({} if overlap else {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9}),
                     **({} if fused else {"merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9})},
         "peak_mem_gb": peak_mem / 1e9,
         "roofline": {

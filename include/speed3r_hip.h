@@ -66,8 +66,9 @@ int s3r_pool_mean(const void* x, void* y, int B, int H, int64_t N, int D, int bl
  * s3r_topk_rows() on `scores` reproduces `topk_idx` bit for bit.  When `scores` is NULL the
  * scores never reach HBM: the attention output comes from a dense sweep of the selection
  * kernel and the indices from a top-k-only kernel that recomputes the scores on chip
- * (bf16/fp16, D == 64, K in {1,2,4,8,16,32}; two launches on `stream`).  `o` may be NULL when
- * only the indices are wanted (MFMA path), `topk_idx` may be NULL when only the attention is.
+ * (bf16/fp16, D == 64, K in {1,2,4,8,16,32}, Lk <= 2^21; two launches on `stream`).  `o` (and then `v`)
+ * may be NULL when only the indices are wanted (MFMA path), `topk_idx` may be NULL when only the
+ * attention is: a caller with two streams runs the two halves side by side.
  * Requires D <= 64 (D == 64 for the MFMA path), K a power of two <= 64.
  */
 int s3r_compressed_attn_topk(const void* q, const void* k, const void* v,

@@ -33,7 +33,7 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
                                         int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
                                         int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t som,
                                         float softmax_scale, int dtype, void* stream) {
-  if (!q || !k || !v || (!o && !topk_idx)) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: null pointer");
+  if (!q || !k || (!o && !topk_idx) || (o && !v)) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: null pointer");
   if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || D <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk: non-positive size");
   if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: dtype %d", dtype);
   if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: head_dim %d > 64", D);
@@ -49,7 +49,7 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
 
   const int es = elt_size(dtype);
   const bool mfma_ok = dtype != S3R_F32 && D == 64 && softmax_scale > 0.f && vec_ok(q, es, sqb, sqh, sqm) &&
-                       vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, som);
+                       vec_ok(k, es, skb, skh, skn) && (!o || (vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, som)));
   if (mfma_ok) return launch_compressed_mfma(p, dtype, stream);
   if (topk_idx != nullptr && scores == nullptr)
     return fail(S3R_ERR_UNSUPPORTED,

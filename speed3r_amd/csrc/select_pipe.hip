@@ -58,6 +58,9 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   const int qb = qg * 4 + wave;
   if (qb >= nqb) return;
 
+#ifdef PROBE_TIMES
+  uint64_t T[8]; T[0] = __builtin_readcyclecounter();
+#endif
   const int64_t N = p.Lq;
   const int64_t q0 = (int64_t)qb * 64;
   const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
@@ -94,6 +97,9 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
     n_full = __popcll(todo);
   }
+#ifdef PROBE_TIMES
+  T[1] = __builtin_readcyclecounter();
+#endif
   if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
@@ -398,10 +404,17 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     dma_v(H0{}, s0);
     int64_t s1 = pop_or_last(), s2 = pop_or_last();
     // the row maxima over the first half tile become the softmax reference; st[.][0] stays for the first phase
+#ifdef PROBE_TIMES
+  T[2] = __builtin_readcyclecounter();
+#endif
     __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the first K half
     scores_half(H0{});
     reads_done();
     dma_k(H0{}, s1);  // the K half the second phase reads
+#ifdef PROBE_TIMES
+  T[3] = __builtin_readcyclecounter();
+#endif
+
     dma_v(H1{}, s0);
     m_i[0] = half_max(st[0][0]);
     m_i[1] = half_max(st[1][0]);
@@ -419,6 +432,9 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
         for (int e = 0; e < 8; e++) vfr[jj][dt][e] = (E)0.f;
+#ifdef PROBE_TIMES
+  T[4] = __builtin_readcyclecounter();
+#endif
     for (int i = n_full; i > 0; i--) {  // past the end of the list the transfers re-read the last tile
       phase(H0{}, s1, s1);
       phase(H1{}, s2, s1);
@@ -426,6 +442,9 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
       s2 = pop_or_last();
     }
     pv_half(H1{});  // PV of the last unit
+#ifdef PROBE_TIMES
+  T[5] = __builtin_readcyclecounter();
+#endif
     // a reference that was too low shows up as a huge or non-finite row sum
     const float big = 1.2676506e30f;  // 2^100
     redo = __any(!(l_i[0] < big) || !(l_i[1] < big));
@@ -500,9 +519,21 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
           }
         }
       }
+#ifndef PROBE_TIMES
     if (live && p.lse != nullptr && hh == 0)
       p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+#endif
   }
+#ifdef PROBE_TIMES
+  T[6] = __builtin_readcyclecounter();
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  T[7] = __builtin_readcyclecounter();
+  if (p.lse != nullptr && lane == 0 && q0 + 8 <= N) {
+    float* dst = p.lse + ((int64_t)b * p.H + h) * N + q0;
+    for (int i = 1; i <= 7; i++) dst[i] = (float)(T[i] - T[0]);
+    dst[0] = (float)(T[0] & 0xffffff);
+  }
+#endif
 }
 
 }  // namespace pipe

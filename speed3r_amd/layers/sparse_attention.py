@@ -96,14 +96,24 @@ class SparseFlashAttentionRope(nn.Module):
         q_c, k_c, v_c = ops.pool_qkv_packed(qkv, h, block)
         pos_c = block_positions(xpos, block) if (xpos is not None and self.rope is not None) else None
         q_c, k_c = self._norm_rope(q_c, self.q_norm, pos_c), self._norm_rope(k_c, self.k_norm, pos_c)
-        o_c, idx = flash_attn_topk_func(q_c, k_c, v_c, self.topk)
-        if self.keep_topk_idx:
-            self.last_topk_idx = idx
+        # the index kernel needs pooled q and k only and its result is first read by the selection kernel: where
+        # it is a kernel of its own it runs on a second stream, beside the compressed attention and the
+        # (HBM-bound) norm/RoPE of the full tokens
+        side = x.is_cuda and ops._two_kernel_compressed(q_c, self.topk)
+        if side:
+            idx, join = ops.topk_indices_on_side_stream(q_c, k_c, self.topk)
+            o_c, _ = ops.compressed_attn_topk(q_c, k_c, v_c, None)
+        else:
+            o_c, idx = flash_attn_topk_func(q_c, k_c, v_c, self.topk)
 
         # selection branch on the full tokens (strided views of the projection; norm/RoPE make q, k contiguous)
         q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)   # each [B, H, N, D]
         pos = xpos if (xpos is not None and self.rope is not None) else None
         q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
+        if side:
+            join()
+        if self.keep_topk_idx:
+            self.last_topk_idx = idx
 
         out = ops.select_attn_merge(q, k, v, idx, o_c, gate, block)
         if out is None:

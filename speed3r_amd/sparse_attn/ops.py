@@ -79,7 +79,7 @@ def pool_qkv_packed(qkv: torch.Tensor, num_heads: int, block: int) -> Tuple[torc
     return y[:, :num_heads], y[:, num_heads:2 * num_heads], y[:, 2 * num_heads:]
 
 
-def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk: Optional[int],
+def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], topk: Optional[int],
                          softmax_scale: Optional[float] = None, return_scores: bool = False,
                          return_lse: bool = False, materialize_scores: Optional[bool] = None):
     """Dense attention over pooled tokens plus, if ``topk`` is given, the top-k columns of the
@@ -90,7 +90,17 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk
     default the selection is fused into the attention kernel wherever the library has it (bf16/fp16,
     head_dim 64, top-k a power of two up to 32): the scores never leave the chip.  Otherwise the scores
     go through HBM (attention kernel, then the row-wise top-k kernel).
+
+    ``v=None`` asks for the indices alone (``o`` is returned as ``None``; fused selection only): the
+    attention output and the indices come from two different kernels, and a caller with two streams runs
+    them side by side, see :func:`sparse_global_attention`.
     """
+    indices_only = v is None
+    if indices_only:
+        assert topk and not return_scores and not return_lse and materialize_scores is not True, \
+            "v=None (indices only) needs top-k without a score buffer"
+        v = k
+        materialize_scores = False
     _need_device(q, k, v)
     _forward_only(q, k, v)
     q, k, v = (_last_contig(t) for t in (q, k, v))
@@ -99,9 +109,10 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk
     lk = k.shape[2]
     assert k.shape == (b, h, lk, d) and v.shape == (b, h, lk, d), "k/v shape mismatch"
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    o = torch.empty_like(q, memory_format=torch.contiguous_format)
+    o = None if indices_only else torch.empty_like(q, memory_format=torch.contiguous_format)
     idx = torch.empty((b, h, lq, topk), dtype=torch.int32, device=q.device) if topk else None
-    fused_ok = (q.dtype != torch.float32 and d == 64 and topk in (1, 2, 4, 8, 16, 32) and _lib.lib_has_fused_topk())
+    fused_ok = (q.dtype != torch.float32 and d == 64 and topk in (1, 2, 4, 8, 16, 32) and lk <= (1 << 21)
+                and _lib.lib_has_fused_topk())
     want_scores = return_scores or (materialize_scores is True) or (
         bool(topk) and materialize_scores is None and not fused_ok)
     if materialize_scores is False and topk and not fused_ok:
@@ -110,13 +121,13 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, topk
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=q.device) if return_lse else None
     with torch.cuda.device(q.device):
         rc = _lib.lib().s3r_compressed_attn_topk(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+            q.data_ptr(), k.data_ptr(), None if indices_only else v.data_ptr(), None if indices_only else o.data_ptr(),
             lse.data_ptr() if lse is not None else None,
             idx.data_ptr() if idx is not None else None,
             scores.data_ptr() if scores is not None else None,
             b, h, lq, lk, d, topk or 0,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), *((0, 0, 0) if indices_only else (o.stride(0), o.stride(1), o.stride(2))),
             scale, _code(q), _stream(q))
     _lib.check(rc, "s3r_compressed_attn_topk")
     out = [o, idx]
@@ -269,23 +280,89 @@ def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: to
     return out
 
 
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority), created on first use and kept."""
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
+
+
+def _two_kernel_compressed(q: torch.Tensor, topk: int) -> bool:
+    """True where the compressed branch is two independent kernels (attention, indices without a score buffer)."""
+    return (q.dtype != torch.float32 and q.shape[-1] == 64 and topk in (1, 2, 4, 8, 16, 32)
+            and q.shape[2] <= (1 << 21) * 64 and _lib.lib_has_fused_topk())
+
+
+def topk_indices_on_side_stream(qc: torch.Tensor, kc: torch.Tensor, topk: int, softmax_scale: Optional[float] = None):
+    """Launch the index kernel (top-k columns of the raw scores ``qc kc^T``, no score buffer) on the device's side
+    stream, ordered after the work already queued on the current stream.  Returns ``(idx, join)``; call ``join()``
+    on the current stream before the first use of ``idx`` there.  Needs :func:`_two_kernel_compressed`."""
+    main = torch.cuda.current_stream(qc.device)
+    side = _side_stream(qc.device)
+    ready = torch.cuda.Event()
+    ready.record(main)
+    side.wait_event(ready)
+    with torch.cuda.stream(side):
+        _, idx = compressed_attn_topk(qc, kc, None, topk, softmax_scale)
+        done = torch.cuda.Event()
+        done.record(side)
+
+    def join():
+        torch.cuda.current_stream(qc.device).wait_event(done)
+        idx.record_stream(torch.cuda.current_stream(qc.device))
+
+    return idx, join
+
+
 def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
                             block: int = 64, topk: int = 16, softmax_scale: Optional[float] = None,
                             return_parts: bool = False, materialize_scores: Optional[bool] = None,
-                            fuse_merge: bool = True):
+                            fuse_merge: bool = True, overlap: bool = False, timeline: Optional[dict] = None):
     """The whole path on post-norm/RoPE q, k, v ``[B,H,N,D]`` and gate ``[B,H,N,2]``:
     pool -> compressed attention + top-k -> selection attention -> gated merge -> ``[B,N,H*D]``.
     The merge runs in the selection kernel's epilogue where the library offers it (same bits either way);
     ``return_parts`` needs the selection output and therefore runs the two operators separately.
+
+    ``overlap``: the indices need pooled q and k only, the compressed attention output is not read before the
+    merge.  Where the two come from different kernels, the index kernel runs on a second stream next to the
+    pooling of v and the compressed attention (same kernels, same results; only the schedule differs).  Measured at
+    266 496 tokens this schedule gains nothing here (the kernels fill the chip one by one), so it is off by default;
+    the layer module uses the same mechanism to hide the index kernel behind the HBM-bound norm/RoPE of the full tokens.
+
+    ``timeline``: a dict that receives timing events of the calling stream under "start", "pooled" (sequential
+    schedule only), "select" (everything before the selection kernel is done) and "end".
     """
-    qc, kc, vc = pool_mean(q, block), pool_mean(k, block), pool_mean(v, block)
-    o_cmp, idx = compressed_attn_topk(qc, kc, vc, topk, softmax_scale, materialize_scores=materialize_scores)
+    def mark(name):
+        if timeline is not None:
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record(torch.cuda.current_stream(q.device))
+            timeline[name] = ev
+
+    mark("start")
+    if overlap and materialize_scores is not True and _two_kernel_compressed(q, topk) and q.is_cuda:
+        qc, kc = pool_mean(q, block), pool_mean(k, block)
+        idx, join = topk_indices_on_side_stream(qc, kc, topk, softmax_scale)
+        vc = pool_mean(v, block)
+        o_cmp, _ = compressed_attn_topk(qc, kc, vc, None, softmax_scale)
+        join()
+    else:
+        qc, kc, vc = pool_mean(q, block), pool_mean(k, block), pool_mean(v, block)
+        mark("pooled")
+        o_cmp, idx = compressed_attn_topk(qc, kc, vc, topk, softmax_scale, materialize_scores=materialize_scores)
+    mark("select")
     if fuse_merge and not return_parts:
         out = select_attn_merge(q, k, v, idx, o_cmp, gate, block, softmax_scale)
         if out is not None:
+            mark("end")
             return out
     o_sel = select_attn(q, k, v, idx, block, softmax_scale)
+    mark("merge")
     out = gated_merge(o_cmp, o_sel, gate, block)
+    mark("end")
     if return_parts:
         return out, dict(idx=idx, o_cmp=o_cmp, o_sel=o_sel, qc=qc, kc=kc, vc=vc)
     return out

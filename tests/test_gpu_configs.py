@@ -71,6 +71,20 @@ def cfg3():
     return cfg, q.to(DEV), k.to(DEV), v.to(DEV), gate.to(DEV)
 
 
+def test_two_stream_schedule_gives_the_same_bits(cfg3):
+    # the index kernel on a second stream beside pooling of v and the compressed attention: same kernels, same
+    # results; repeated, so that an ordering hole between the streams would have a chance to show
+    cfg, q, k, v, gate = cfg3
+    want = s3r.sparse_global_attention(q, k, v, gate, 64, cfg.topk, overlap=False)
+    for _ in range(4):
+        got = s3r.sparse_global_attention(q, k, v, gate, 64, cfg.topk, overlap=True)
+        assert torch.equal(got, want)
+    qc, kc = s3r.pool_mean(q, 64), s3r.pool_mean(k, 64)
+    _, idx_seq = s3r.compressed_attn_topk(qc, kc, s3r.pool_mean(v, 64), cfg.topk)
+    none, idx_only = s3r.compressed_attn_topk(qc, kc, None, cfg.topk)
+    assert none is None and torch.equal(idx_only, idx_seq)
+
+
 def test_config3_full_size_properties(cfg3):
     cfg, q, k, v, gate = cfg3
     n, nc = cfg.tokens, cfg.tokens // 64
