@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[4 * kHalf * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[4 * kHalf * 2];
 
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int lane = threadIdx.x & 63;
   const int hh = lane >> 5;
   const int c = lane & 31;
@@ -80,6 +80,28 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   typedef std::integral_constant<int, 0> H0;
   typedef std::integral_constant<int, 1> H1;
 
+  // Q block -> LDS by direct transfers (the two V half buffers hold it until the first V tile is fetched), in the
+  // layout of a K tile, so that the B operands are read like K fragments.  Lane-linear transfers cost the texture
+  // path a quarter of what operand-pattern global loads cost.  Rows beyond N re-read the last row (never stored).
+  {
+    const int qr = lane >> 3;
+    const uint32_t q_chunk = (uint32_t)(((lane & 7) ^ (qr & 7)) * 8 * (int)sizeof(E));
+    const uint32_t q_rowbytes = (uint32_t)p.sqm * (uint32_t)sizeof(E);
+    const int q_last = (int)((N - q0 < 64 ? N - q0 : 64) - 1);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + q0 * p.sqm), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      char* dst = reinterpret_cast<char*>(qt == 0 ? v_half(H0{}) : v_half(H1{}));
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        int row = 32 * qt + 8 * i + qr;
+        row = row < q_last ? row : q_last;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16,
+                                                 (uint32_t)row * q_rowbytes + q_chunk, 0, 0, 0);
+      }
+    }
+  }
+
   // index list: full tiles go through the pipeline, occurrences of the ragged last block come after it
   int32_t my_idx = -1;
   const int32_t ragged_blk = (N & 63) ? (int32_t)(N >> 6) : -1;
@@ -101,6 +123,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   T[1] = __builtin_readcyclecounter();
 #endif
   if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer may still write LDS when the wave ends
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
       const int64_t row = q0 + qt * 32 + c;
@@ -114,17 +137,6 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   }
 
   V8 bq[2][4];
-#pragma unroll
-  for (int qt = 0; qt < 2; qt++) {
-    const int64_t row = q0 + qt * 32 + c;
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      Frag f;
-      f.u = make_uint4(0, 0, 0, 0);
-      if (row < N) f.u = *reinterpret_cast<const uint4*>(qp + row * p.sqm + ks * 16 + hh * 8);
-      bq[qt][ks] = as_v8<E>(f);
-    }
-  }
 
   f32x16 ot[2][2];  // [dt][qt]
 #pragma unroll
@@ -382,6 +394,47 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   };
 
   bool redo = false;
+  // Operands of the gated merge (epilogue): gate pair per query row, the query block's row of the compressed output
+  // in this lane's store layout.  Issued right after the main loop, so that their latency passes behind the last PV
+  // stage instead of in front of the stores.
+  const bool merge = p.merge_out != nullptr;
+  float g0[2] = {0.f, 0.f}, g1[2] = {0.f, 0.f};
+  uint4 oc_raw[2][2];  // [dt][gp]
+  bool merge_loaded = false;
+  auto load_merge_operands = [&]() {
+    if (merge) {
+#pragma unroll
+      for (int qt = 0; qt < 2; qt++) {
+        const int64_t row = q0 + qt * 32 + c;
+        if (row < N) {
+          const E* gp = (const E*)p.merge_gate + (int64_t)b * p.sgb + (int64_t)h * p.sgh + row * p.sgn;
+          g0[qt] = (float)gp[0];
+          g1[qt] = (float)gp[1];
+        }
+      }
+      const E* ocp = (const E*)p.merge_oc + (int64_t)b * p.scb + (int64_t)h * p.sch + (int64_t)qb * p.scm;
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int gp = 0; gp < 2; gp++) oc_raw[dt][gp] = *reinterpret_cast<const uint4*>(ocp + dt * 32 + 8 * (2 * gp + hh));
+    }
+    merge_loaded = true;
+  };
+
+  {  // B operands from the staged Q block: lane = query row, head_dim chunk hh + 2*ks
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the Q transfers have landed
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      const char* qbase = reinterpret_cast<const char*>(qt == 0 ? v_half(H0{}) : v_half(H1{}));
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(qbase + (kr_off ^ (ks << 5)));
+        bq[qt][ks] = as_v8<E>(f);
+      }
+    }
+    reads_done();  // before the V buffers are refilled
+  }
   if (n_full > 0) {
     int64_t last_start = 0;
     auto pop_or_last = [&]() -> int64_t {  // branch-free: next full tile, or the last one again
@@ -441,6 +494,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
       s1 = s2;
       s2 = pop_or_last();
     }
+    load_merge_operands();
     pv_half(H1{});  // PV of the last unit
 #ifdef PROBE_TIMES
   T[5] = __builtin_readcyclecounter();
@@ -469,7 +523,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   // Output: lane (c, hh) holds for query c + 32*qt the head_dim values dt*32 + 8*g4 + 4*hh + {0..3}.  One exchange with
   // lane ^ 32 per packed word hands every lane eight consecutive head_dim values (hh = 0: group g4 = 2*gp, hh = 1:
   // group 2*gp + 1), so a row receives 32 contiguous bytes per store instruction.
-  const bool merge = p.merge_out != nullptr;
+  if (!merge_loaded) load_merge_operands();
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
 #pragma clang fp contract(off)  // the merge rounds each product and the sum separately, like the eager expression
@@ -477,12 +531,6 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     const float inv = l > 0.f ? 1.f / l : 0.f;
     const int64_t row = q0 + qt * 32 + c;
     const bool live = row < N;
-    float g0 = 0.f, g1 = 0.f;
-    if (merge && live) {
-      const E* gp = (const E*)p.merge_gate + (int64_t)b * p.sgb + (int64_t)h * p.sgh + row * p.sgn;
-      g0 = (float)gp[0];
-      g1 = (float)gp[1];
-    }
 #pragma unroll
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -508,11 +556,11 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
             *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
           } else {
             union { E e[8]; uint4 u; } oc, res;
-            oc.u = *reinterpret_cast<const uint4*>((const E*)p.merge_oc + (int64_t)b * p.scb + (int64_t)h * p.sch + (int64_t)qb * p.scm + d0);
+            oc.u = oc_raw[dt][gp];
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-              const float x = round_to<E>(g0 * (float)oc.e[e]);
-              const float y = round_to<E>(g1 * (float)pc.e[e]);
+              const float x = round_to<E>(g0[qt] * (float)oc.e[e]);
+              const float y = round_to<E>(g1[qt] * (float)pc.e[e]);
               res.e[e] = (E)(x + y);
             }
             *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = res.u;
