@@ -30,17 +30,21 @@ namespace pipe {
 using namespace sel;
 
 constexpr int kHalf = 32 * 64;  // elements per half tile
+#ifndef S3R_PIPE_WAVES
+#define S3R_PIPE_WAVES 4
+#endif
+constexpr int kWaves = S3R_PIPE_WAVES;  // wavefronts (= query blocks) per workgroup; the waves do not interact
 
 // DENSE: no index list, every query block attends to all key tiles in order (the compressed branch's attention over
 // the pooled tokens runs through this instance).
 template <typename E, bool DENSE>
-__global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
+__global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[4 * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[4 * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[4 * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[4 * kHalf * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[kWaves * kHalf * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[kWaves * kHalf * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kWaves * kHalf * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kWaves * kHalf * 2];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int lane = threadIdx.x & 63;
@@ -55,7 +59,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
   const int qg = vid - bh * nqg;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
-  const int qb = qg * 4 + wave;
+  const int qb = qg * kWaves + wave;
   if (qb >= nqb) return;
 
 #ifdef PROBE_TIMES
@@ -113,7 +117,27 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     n_full = (int)(N >> 6);
     n_ragged = (N & 63) ? 1 : 0;
   } else {
-    my_idx = lane < p.K ? idx_row[lane] : -1;
+    // The list comes through the scalar cache (s_load): a vector load would wait in the vector memory queue behind
+    // the Q transfers and behind the other waves' tile transfers, and the first K transfer waits for the list.
+    const int32_t __attribute__((address_space(4)))* srow = (const int32_t __attribute__((address_space(4)))*)idx_row;
+    if (p.K == 16) {
+      int32_t sidx[16];
+#pragma unroll
+      for (int i = 0; i < 16; i++) sidx[i] = srow[i];
+#pragma unroll
+      for (int i = 0; i < 16; i++) my_idx = lane == i ? sidx[i] : my_idx;
+    } else if (p.K == 32) {
+      int32_t sidx[32];
+#pragma unroll
+      for (int i = 0; i < 32; i++) sidx[i] = srow[i];
+#pragma unroll
+      for (int i = 0; i < 32; i++) my_idx = lane == i ? sidx[i] : my_idx;
+    } else {
+      for (int i = 0; i < p.K; i++) {  // other lengths: one entry at a time
+        const int32_t v = srow[i];
+        my_idx = lane == i ? v : my_idx;
+      }
+    }
     my_valid = my_idx >= 0 && (int64_t)my_idx * 64 < N;
     todo = __ballot(my_valid && my_idx != ragged_blk);
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
@@ -421,8 +445,7 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     merge_loaded = true;
   };
 
-  {  // B operands from the staged Q block: lane = query row, head_dim chunk hh + 2*ks
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the Q transfers have landed
+  auto read_q = [&]() {  // B operands from the staged Q block: lane = query row, head_dim chunk hh + 2*ks
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
       const char* qbase = reinterpret_cast<const char*>(qt == 0 ? v_half(H0{}) : v_half(H1{}));
@@ -434,6 +457,10 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
       }
     }
     reads_done();  // before the V buffers are refilled
+  };
+  if (n_full == 0) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the Q transfers have landed
+    read_q();
   }
   if (n_full > 0) {
     int64_t last_start = 0;
@@ -454,6 +481,8 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
     // transfers in the rotation of the loop (K1, V0, K0, V1), so that the loop's waits hold from the first phase on
     dma_k(H0{}, s0);
     dma_k(H1{}, s0);
+    __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the Q transfers, issued before these eight, have landed
+    read_q();
     dma_v(H0{}, s0);
     int64_t s1 = pop_or_last(), s2 = pop_or_last();
     // the row maxima over the first half tile become the softmax reference; st[.][0] stays for the first phase
@@ -588,11 +617,11 @@ __global__ __launch_bounds__(256, 2) void select_pipe_kernel(AttnParams p, int n
 
 int launch_select_pipe(const AttnParams& p, int dtype, void* stream) {
   const int64_t nqb = (p.Lq + 63) / 64;
-  const int64_t nqg = (nqb + 3) / 4;
+  const int64_t nqg = (nqb + pipe::kWaves - 1) / pipe::kWaves;
   const int64_t total = nqg * p.B * p.H;
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)total), blk(256);
+  dim3 grid((unsigned)total), blk(64 * pipe::kWaves);
   const bool dense = p.idx == nullptr;  // no index list: every query block sweeps all key tiles
   if (dense && p.Lq != p.Lk) return fail(S3R_ERR_UNSUPPORTED, "dense sweep: Lq %lld != Lk %lld", (long long)p.Lq, (long long)p.Lk);
   if (dtype == S3R_BF16) {
