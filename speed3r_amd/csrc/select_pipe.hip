@@ -62,9 +62,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const int qb = qg * kWaves + wave;
   if (qb >= nqb) return;
 
-#ifdef PROBE_TIMES
-  uint64_t T[8]; T[0] = __builtin_readcyclecounter();
-#endif
   const int64_t N = p.Lq;
   const int64_t q0 = (int64_t)qb * 64;
   const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
@@ -143,9 +140,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
     n_full = __popcll(todo);
   }
-#ifdef PROBE_TIMES
-  T[1] = __builtin_readcyclecounter();
-#endif
   if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer may still write LDS when the wave ends
 #pragma unroll
@@ -486,16 +480,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     dma_v(H0{}, s0);
     int64_t s1 = pop_or_last(), s2 = pop_or_last();
     // the row maxima over the first half tile become the softmax reference; st[.][0] stays for the first phase
-#ifdef PROBE_TIMES
-  T[2] = __builtin_readcyclecounter();
-#endif
     __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the first K half
     scores_half(H0{});
     reads_done();
     dma_k(H0{}, s1);  // the K half the second phase reads
-#ifdef PROBE_TIMES
-  T[3] = __builtin_readcyclecounter();
-#endif
 
     dma_v(H1{}, s0);
     m_i[0] = half_max(st[0][0]);
@@ -514,9 +502,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
         for (int e = 0; e < 8; e++) vfr[jj][dt][e] = (E)0.f;
-#ifdef PROBE_TIMES
-  T[4] = __builtin_readcyclecounter();
-#endif
     for (int i = n_full; i > 0; i--) {  // past the end of the list the transfers re-read the last tile
       phase(H0{}, s1, s1);
       phase(H1{}, s2, s1);
@@ -525,9 +510,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     }
     load_merge_operands();
     pv_half(H1{});  // PV of the last unit
-#ifdef PROBE_TIMES
-  T[5] = __builtin_readcyclecounter();
-#endif
     // a reference that was too low shows up as a huge or non-finite row sum
     const float big = 1.2676506e30f;  // 2^100
     redo = __any(!(l_i[0] < big) || !(l_i[1] < big));
@@ -596,21 +578,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
           }
         }
       }
-#ifndef PROBE_TIMES
     if (live && p.lse != nullptr && hh == 0)
       p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-#endif
   }
-#ifdef PROBE_TIMES
-  T[6] = __builtin_readcyclecounter();
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  T[7] = __builtin_readcyclecounter();
-  if (p.lse != nullptr && lane == 0 && q0 + 8 <= N) {
-    float* dst = p.lse + ((int64_t)b * p.H + h) * N + q0;
-    for (int i = 1; i <= 7; i++) dst[i] = (float)(T[i] - T[0]);
-    dst[0] = (float)(T[0] & 0xffffff);
-  }
-#endif
 }
 
 }  // namespace pipe
