@@ -168,6 +168,38 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
                     int64_t sgb, int64_t sgh, int64_t sgn,
                     int dtype, void* stream);
 
+/*
+ * Backward of the two attention operators (bf16/fp16, head_dim 64, block 64).
+ * Replaces _topk_blocksparse_attention_bwd (pi3/models/sparse_attn/topk_blocksparse_attention.py:907-1038, kernels
+ * backward_sum_o_do :132-170, backward_dkdv :558-712, backward_dq :722-850) and, with idx == NULL (every key tile),
+ * _flash_attn_backward (pi3/models/sparse_attn/flash_attention_topk.py:204-630).
+ *
+ * s3r_attn_bwd_delta:  delta[b,h,n] = sum_d o[b,h,n,d] * dout[b,h,n,d]  (fp32, contiguous [B,H,N]).
+ * s3r_attn_bwd: with P = exp(scale * q k^T - lse) over the keys the forward attended to,
+ *   dv = P^T dout,  dS = scale * P * (dout v^T - delta),  dq = dS k,  dk = dS^T q;
+ *   P and dS are rounded to the I/O dtype before the products, accumulation is fp32.
+ *   lse: the forward's optional output (natural log, scaled scores), fp32 [B,H,Lq] contiguous.
+ *   idx: the forward's block indices [B,H,ceil(Lq/64),K] (strides sib,sih,sim), or NULL for dense attention.
+ *   kq_list, kq_off (needed for dk/dv when idx is given): for every (b,h) the query-block ids that list key block j,
+ *     one entry per occurrence, ascending, are kq_list[(b*H+h)*list_stride + kq_off[(b*H+h)*(nkb+1) + j] ...
+ *     kq_off[... + j+1]), nkb = ceil(Lk/64); entries of idx that are < 0 or >= nkb appear in no list
+ *     (reference count_query_fixedlen / reorder_topk_idx_fixedlen, :423-554).
+ *   dq (layout strides sdq*), dk, dv (sdk*, sdv*): I/O dtype; dq == NULL or dk == dv == NULL skips that kernel.
+ *   Every row of dq, dk, dv inside the tensors is written (zeros where nothing attends).
+ */
+int s3r_attn_bwd_delta(const void* o, const void* dout, float* delta, int B, int H, int64_t N, int D,
+                       int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
+                       int dtype, void* stream);
+int s3r_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse, const float* delta,
+                 const int32_t* idx, const int32_t* kq_list, const int32_t* kq_off, int64_t list_stride,
+                 void* dq, void* dk, void* dv,
+                 int B, int H, int64_t Lq, int64_t Lk, int D, int block, int K,
+                 int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
+                 int64_t svb, int64_t svh, int64_t svn, int64_t sgb, int64_t sgh, int64_t sgm,
+                 int64_t sdqb, int64_t sdqh, int64_t sdqm, int64_t sdkb, int64_t sdkh, int64_t sdkn,
+                 int64_t sdvb, int64_t sdvh, int64_t sdvn, int64_t sib, int64_t sih, int64_t sim,
+                 float softmax_scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

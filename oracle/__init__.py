@@ -19,3 +19,10 @@ from .sparse_attention_oracle import (  # noqa: F401
     sparse_global_attention,
 )
 from .sparse_layer_oracle import rope2d, block_positions, sparse_layer  # noqa: F401,E402
+from .attention_grad_oracle import (  # noqa: F401,E402
+    select_attention_grads_autograd,
+    compressed_attention_grads_autograd,
+    attention_grads_formula,
+    block_multiplicity,
+    key_block_lists,
+)

@@ -1,6 +1,7 @@
 // C-ABI entry points of the two attention operators: argument validation and kernel choice.
 #include "s3r_common.h"
 #include "attn_params.h"
+#include "attn_bwd.h"
 #include <stdlib.h>
 #include <string.h>
 
@@ -141,4 +142,49 @@ extern "C" int s3r_select_attn_merge(const void* q, const void* k, const void* v
   const MergeArgs m = {o_cmp, gate, out, scb, sch, scm, sgb, sgh, sgn};
   return select_attn_impl("s3r_select_attn_merge", q, k, v, idx, nullptr, nullptr, B, H, N, D, block, K, sqb, sqh, sqn,
                           skb, skh, skn, svb, svh, svn, 0, 0, 0, sib, sih, sim, softmax_scale, dtype, m, stream);
+}
+
+extern "C" int s3r_attn_bwd_delta(const void* o, const void* dout, float* delta, int B, int H, int64_t N, int D,
+                                  int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
+                                  int dtype, void* stream) {
+  if (!o || !dout || !delta) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd_delta: null pointer");
+  if (B <= 0 || H <= 0 || N <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd_delta: non-positive size");
+  if ((dtype != S3R_BF16 && dtype != S3R_F16) || D != 64)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd_delta: built for bf16/fp16, head_dim 64");
+  if (!vec_ok(o, 2, sob, soh, son) || !vec_ok(dout, 2, sdb, sdh, sdn))
+    return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd_delta: pointers and strides must be multiples of 16 bytes");
+  return launch_bwd_delta(o, dout, delta, B, H, N, sob, soh, son, sdb, sdh, sdn, dtype, stream);
+}
+
+extern "C" int s3r_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse, const float* delta,
+                            const int32_t* idx, const int32_t* kq_list, const int32_t* kq_off, int64_t list_stride,
+                            void* dq, void* dk, void* dv,
+                            int B, int H, int64_t Lq, int64_t Lk, int D, int block, int K,
+                            int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
+                            int64_t svb, int64_t svh, int64_t svn, int64_t sgb, int64_t sgh, int64_t sgm,
+                            int64_t sdqb, int64_t sdqh, int64_t sdqm, int64_t sdkb, int64_t sdkh, int64_t sdkn,
+                            int64_t sdvb, int64_t sdvh, int64_t sdvn, int64_t sib, int64_t sih, int64_t sim,
+                            float softmax_scale, int dtype, void* stream) {
+  if (!q || !k || !v || !dout || !lse || !delta) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: null pointer");
+  if (!dq && !dk && !dv) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: no gradient requested");
+  if ((dk == nullptr) != (dv == nullptr)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: dk and dv come together");
+  if (idx != nullptr && dk != nullptr && (!kq_list || !kq_off)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: dk/dv of the selection branch need the key-centric lists");
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || (idx != nullptr && K <= 0)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: non-positive size");
+  if ((dtype != S3R_BF16 && dtype != S3R_F16) || D != 64 || block != 64 || K > 64 || !(softmax_scale > 0.f))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd: built for bf16/fp16, head_dim 64, block 64, top-k <= 64, positive scale");
+  const int64_t lim = 1 << 20;
+  if (sqm <= 0 || skn <= 0 || svn <= 0 || sgm <= 0 || sqm >= lim || skn >= lim || svn >= lim || sgm >= lim)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd: row strides must be positive and below 2^20 elements");
+  if (!vec_ok(q, 2, sqb, sqh, sqm) || !vec_ok(k, 2, skb, skh, skn) || !vec_ok(v, 2, svb, svh, svn) || !vec_ok(dout, 2, sgb, sgh, sgm) ||
+      (dq && !vec_ok(dq, 2, sdqb, sdqh, sdqm)) || (dk && (!vec_ok(dk, 2, sdkb, sdkh, sdkn) || !vec_ok(dv, 2, sdvb, sdvh, sdvn))))
+    return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: pointers and strides must be multiples of 16 bytes");
+  BwdParams p = {};
+  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.idx = idx; p.kq_list = kq_list; p.kq_off = kq_off; p.list_stride = list_stride;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.K = K;
+  p.sqb = sqb; p.sqh = sqh; p.sqm = sqm; p.skb = skb; p.skh = skh; p.skn = skn; p.svb = svb; p.svh = svh; p.svn = svn;
+  p.sgb = sgb; p.sgh = sgh; p.sgm = sgm; p.sdqb = sdqb; p.sdqh = sdqh; p.sdqm = sdqm; p.sdkb = sdkb; p.sdkh = sdkh; p.sdkn = sdkn;
+  p.sdvb = sdvb; p.sdvh = sdvh; p.sdvn = sdvn; p.sib = sib; p.sih = sih; p.sim = sim;
+  p.scale = softmax_scale;
+  return launch_attn_bwd(p, dtype, stream);
 }

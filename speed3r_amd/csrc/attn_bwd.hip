@@ -1,0 +1,513 @@
+// Backward of the two attention operators on the gfx950 matrix cores (bf16 / fp16 I/O, block 64, head_dim 64).
+//
+// Reference: _topk_blocksparse_attention_bwd with backward_sum_o_do, backward_dkdv, backward_dq
+// (pi3/models/sparse_attn/topk_blocksparse_attention.py:132-170,558-712,722-850,907-1038) for the selection
+// branch and _flash_attn_backward (pi3/models/sparse_attn/flash_attention_topk.py:204-630) for the compressed
+// branch, which is the same computation over ALL key tiles (DENSE below).  With P = exp(scale*S - lse) recomputed
+// from the forward's log-sum-exp and delta = rowsum(dO * O):
+//   dV = P^T dO          dP = dO V^T          dS = scale * P * (dP - delta)          dQ = dS K          dK = dS^T Q
+// P (for dV) and dS (for dQ, dK) are rounded to the I/O dtype before the products, accumulation is fp32
+// (reference :683-690, :826-838).
+//
+// Three kernels:
+//   * bwd_delta_kernel: delta[b,h,n] = sum_d o * dO in fp32 (HBM bound).
+//   * bwd_dq_kernel: one wavefront per 64-row query block, four independent waves per workgroup; walks the block's
+//     selected key tiles (or all of them).  Everything is computed transposed, as in the forward kernels:
+//     S^T = K Q^T and dP^T = V dO^T put one QUERY per lane, so lse and delta are per-lane scalars;
+//     dQ^T += K^T dS^T takes K^T fragments from ds_read_b64_tr_b16.  K and V half tiles (32 keys) go global -> LDS
+//     by direct transfers, double buffered (16 KB per wave).  The K half is staged once, in the layout of the
+//     transposed reads; its row reads (A operand of S^T) then take a 2-way bank conflict.
+//   * bwd_dkdv_kernel: one workgroup of two waves per 64-key block, each wave owns 32 keys (one KEY per lane:
+//     S = Q K^T, dP = dO V^T with K, V fragments in registers as B operands) and walks the query blocks that
+//     selected the key block (key-centric lists built by the host from the index tensor, reference :423-554).
+//     Q and dO half tiles (32 queries) and the matching lse / delta values go global -> LDS, shared by the two
+//     waves, double buffered, one barrier per half tile; dV^T += dO^T P and dK^T += Q^T dS read their A operands
+//     transposed from the same buffers.
+// Query rows beyond Lq have lse = +inf (P = 0), keys beyond Lk are masked (P = 0); rows past the end of a tensor are
+// never read (transfers re-read the last valid row).
+#include "select_common.h"
+#include "attn_bwd.h"
+
+namespace s3r {
+namespace bwd {
+using namespace sel;
+
+constexpr int kHalfBytes = 32 * 128;  // one half tile: 32 rows of 64 two-byte values
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef std::integral_constant<int, 0> H0;
+typedef std::integral_constant<int, 1> H1;
+
+// ---- delta ---------------------------------------------------------------------------------------------------
+template <typename E>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const E* __restrict__ o, const E* __restrict__ dout, float* __restrict__ delta,
+                                                         int H, int64_t N, int64_t rows, int64_t sob, int64_t soh, int64_t son,
+                                                         int64_t sdb, int64_t sdh, int64_t sdn) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = gid >> 3;  // 8 lanes of 16 bytes per 64-value row
+  const int part = (int)(gid & 7);
+  const bool live = row < rows;
+  const int64_t rr = live ? row : rows - 1;
+  const int64_t n = rr % N, bh = rr / N;
+  const int h = (int)(bh % H);
+  const int64_t b = bh / H;
+  const uint4 a = *reinterpret_cast<const uint4*>(o + b * sob + h * soh + n * son + part * 8);
+  const uint4 g = *reinterpret_cast<const uint4*>(dout + b * sdb + h * sdh + n * sdn + part * 8);
+  const E* ae = reinterpret_cast<const E*>(&a);
+  const E* ge = reinterpret_cast<const E*>(&g);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) s += (float)ae[i] * (float)ge[i];
+#pragma unroll
+  for (int off = 1; off < 8; off <<= 1) s += __shfl_xor(s, off);
+  if (live && part == 0) delta[rr] = s;
+}
+
+// ---- shared pieces of the two MFMA kernels -----------------------------------------------------------------------
+// Transfer of rows [8*i0*.., ...) of a 32-row half tile: instruction i moves rows 8i .. 8i+7 (16 bytes per lane).
+// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ (((row>>1)&1)<<2) (layout of the transposed reads), else
+// c' ^ (row&7) (layout of conflict-free row reads).  Rows are clamped to `last` (relative to `base`'s row 0).
+template <typename E, bool VSW>
+__device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int first_row, int last, char* lds_half, int lane, int i_begin, int i_end) {
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
+  const int lr = lane >> 3;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if (i >= i_begin && i < i_end) {
+      const int ldsrow = 8 * i + lr;
+      int row = first_row + ldsrow;
+      row = row < last ? row : last;
+      const int chunk = (lane & 7) ^ (VSW ? (((ldsrow >> 1) & 1) << 2) : (ldsrow & 7));
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
+                                               (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
+    }
+  }
+}
+
+// A operand from row reads of a half tile: lane = row c, k-step ks: head_dim chunk 2ks + hh.
+template <typename E, bool VSW>
+__device__ __forceinline__ void read_rows(const char* half, int c, int hh, typename Mma<E>::V8 (&dst)[4]) {
+  const int sw = VSW ? (((c >> 1) & 1) << 2) : (c & 7);
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) {
+    Frag f;
+    f.u = *reinterpret_cast<const uint4*>(half + c * 128 + (((2 * ks + hh) ^ sw) << 4));
+    dst[ks] = as_v8<E>(f);
+  }
+}
+
+// A operand X^T from transposed reads of a half tile staged with VSW: fragment [jj][dt] holds, for head_dim row
+// dt*32 + c, the 8 rows 16jj + {4hh..4hh+3, 8+4hh..8+4hh+3} of the half: the order in which a 32x32 accumulator
+// with one column per lane hands over its registers 8jj .. 8jj+7.
+template <typename E>
+__device__ __forceinline__ void read_transposed(const char* half, int tr_off, typename Mma<E>::V8 (&dst)[2][2]) {
+#pragma unroll
+  for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++) {
+      const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+      Frag f;
+      f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+      f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+      dst[jj][dt] = as_v8<E>(f);
+    }
+}
+
+__device__ __forceinline__ int tr_offset(int lane) {
+  const int hh = lane >> 5;
+  const int i16 = lane & 15;
+  const int tr_row = 4 * hh + (i16 >> 2);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
+  return tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
+}
+
+// Store of a transposed 64 x 64 accumulator pair acc[dt] (lane = row of the output, registers = head_dim values
+// dt*32 + 8*(r/4) + 4*hh + r%4): one exchange with lane ^ 32 per packed word gives every lane 8 consecutive values.
+template <typename E>
+__device__ __forceinline__ void store_rows(const f32x16 (&acc)[2], E* rowptr, bool live, int hh) {
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int gp = 0; gp < 2; gp++) {
+      union { E e[8]; uint32_t w[4]; uint4 u; } pc;
+      union { E e[2]; uint32_t w; } t;
+#pragma unroll
+      for (int wi = 0; wi < 2; wi++) {
+        t.e[0] = (E)acc[dt][8 * gp + 2 * wi];
+        t.e[1] = (E)acc[dt][8 * gp + 2 * wi + 1];
+        const uint32_t a = t.w;
+        t.e[0] = (E)acc[dt][8 * gp + 4 + 2 * wi];
+        t.e[1] = (E)acc[dt][8 * gp + 4 + 2 * wi + 1];
+        const uint32_t bw = t.w;
+        const auto r = __builtin_amdgcn_permlane32_swap(a, bw, false, false);
+        pc.w[wi] = r[0];
+        pc.w[2 + wi] = r[1];
+      }
+      if (live) *reinterpret_cast<uint4*>(rowptr + dt * 32 + 8 * (2 * gp + hh)) = pc.u;
+    }
+}
+
+// ---- dQ ----------------------------------------------------------------------------------------------------------
+template <typename E, bool DENSE>
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, int nqg, int total_wg) {
+  typedef typename Mma<E>::V8 V8;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[4 * kHalfBytes];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int hh = lane >> 5;
+  const int c = lane & 31;
+
+  const int w = blockIdx.x;  // workgroup w -> work item: each XCD walks a contiguous range of query blocks of one head
+  const int xcd = w & 7, slot = w >> 3;
+  const int per = total_wg >> 3, rem = total_wg & 7;
+  const int vid = xcd * per + (xcd < rem ? xcd : rem) + slot;
+  const int bh = vid / nqg;
+  const int qg = vid - bh * nqg;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+  const int qb = qg * 4 + wave;
+  if (qb >= nqb) return;
+
+  const int64_t Lq = p.Lq, Lk = p.Lk;
+  const int64_t q0 = (int64_t)qb * 64;
+  const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
+  const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
+  const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
+  const E* gp = (const E*)p.dout + (int64_t)b * p.sgb + (int64_t)h * p.sgh;
+  const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
+  const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
+
+  char* k_buf[2] = {reinterpret_cast<char*>(lds_k0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_k1) + wave * kHalfBytes};
+  char* v_buf[2] = {reinterpret_cast<char*>(lds_v0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_v1) + wave * kHalfBytes};
+
+  // B operands Q and dO (lane = query row, head_dim chunk hh + 2 ks), per-query lse (base 2) and delta
+  V8 bq[2][4], bg[2][4];
+  float lse2[2], dlt[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++) {
+    const int64_t row = q0 + qt * 32 + c;
+    const bool live = row < Lq;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      Frag f, g;
+      f.u = make_uint4(0, 0, 0, 0);
+      g.u = make_uint4(0, 0, 0, 0);
+      if (live) {
+        f.u = *reinterpret_cast<const uint4*>(qp + row * p.sqm + ks * 16 + hh * 8);
+        g.u = *reinterpret_cast<const uint4*>(gp + row * p.sgm + ks * 16 + hh * 8);
+      }
+      bq[qt][ks] = as_v8<E>(f);
+      bg[qt][ks] = as_v8<E>(g);
+    }
+    lse2[qt] = live ? lsep[row] * kLog2e : INFINITY;
+    dlt[qt] = live ? dlp[row] : 0.f;
+  }
+  f32x16 dqt[2][2];  // dQ^T accumulators [qt][dt]: lane = query, registers = head_dim
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) dqt[qt][dt][r] = 0.f;
+
+  // key tiles of this query block
+  int32_t my_idx = -1;
+  uint64_t todo = 0;
+  int ntiles;
+  int dense_next = 0;
+  if constexpr (DENSE) {
+    ntiles = (int)((Lk + 63) >> 6);
+  } else {
+    const int32_t* idx_row = p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
+    my_idx = lane < p.K ? idx_row[lane] : -1;
+    todo = __ballot(my_idx >= 0 && (int64_t)my_idx * 64 < Lk);
+    ntiles = __popcll(todo);
+  }
+  auto pop = [&]() -> int64_t {  // start row of the next tile (callers pop exactly ntiles times)
+    if constexpr (DENSE) {
+      return (int64_t)(dense_next++) * 64;
+    } else {
+      const int t = __ffsll((unsigned long long)todo) - 1;
+      todo &= todo - 1;
+      return (int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64;
+    }
+  };
+
+  const float sl2 = p.scale * kLog2e;
+  const uint32_t krow = (uint32_t)p.skn * (uint32_t)sizeof(E), vrow = (uint32_t)p.svn * (uint32_t)sizeof(E);
+  const int tr_off = tr_offset(lane);
+
+  auto fetch = [&](int64_t start, auto hf, int buf) {  // half HF of the tile at `start` -> buffers `buf`
+    constexpr int HF = decltype(hf)::value;
+    const int last = (int)((Lk - start < 64 ? Lk - start : 64) - 1);
+    dma_rows<E, true>(kp + start * p.skn, krow, 32 * HF, last, k_buf[buf], lane, 0, 4);
+    dma_rows<E, false>(vp + start * p.svn, vrow, 32 * HF, last, v_buf[buf], lane, 0, 4);
+  };
+  auto compute = [&](int64_t start, auto hf, int buf) {
+    constexpr int HF = decltype(hf)::value;
+    const int nvalid = (int)(Lk - start < 64 ? Lk - start : 64);
+    const bool ragged = nvalid < 64;
+    V8 ak[4], av[4];
+    read_rows<E, true>(k_buf[buf], c, hh, ak);
+    read_rows<E, false>(v_buf[buf], c, hh, av);
+    V8 ds[2][2];  // dS^T as B operand [qt][jj]
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      f32x16 st, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) { st[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) st = Mma<E>::mma(ak[ks], bq[qt][ks], st);
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(av[ks], bg[qt][ks], dp);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float pv = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));
+        if (ragged && (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid)) pv = 0.f;
+        ds[qt][r >> 3][r & 7] = (E)(pv * (dp[r] - dlt[qt]) * p.scale);
+      }
+    }
+    V8 kt[2][2];
+    read_transposed<E>(k_buf[buf], tr_off, kt);
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int qt = 0; qt < 2; qt++) dqt[qt][dt] = Mma<E>::mma(kt[jj][dt], ds[qt][jj], dqt[qt][dt]);
+  };
+
+  if (ntiles > 0) {
+    int64_t cur = pop();
+    fetch(cur, H0{}, 0);
+    for (int t = 0; t < ntiles; t++) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffer 1 (previous tile) are done
+      fetch(cur, H1{}, 1);
+      __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): half 0 has landed
+      compute(cur, H0{}, 0);
+      const bool more = t + 1 < ntiles;
+      const int64_t nxt = more ? pop() : cur;
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffer 0 are done
+      if (more) {
+        fetch(nxt, H0{}, 0);
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): half 1 has landed
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
+      compute(cur, H1{}, 1);
+      cur = nxt;
+    }
+  }
+
+  E* dqp = (E*)p.dq + (int64_t)b * p.sdqb + (int64_t)h * p.sdqh;
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++) {
+    const int64_t row = q0 + qt * 32 + c;
+    store_rows<E>(dqt[qt], dqp + row * p.sdqm, row < Lq, hh);
+  }
+}
+
+// ---- dK, dV ------------------------------------------------------------------------------------------------------
+template <typename E, bool DENSE>
+__global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, int nqb_all, int total_wg) {
+  typedef typename Mma<E>::V8 V8;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_q0[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_g0[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_g1[kHalfBytes];
+  __shared__ __attribute__((aligned(256))) float lds_s0[128];  // [0,64): lse of the half's 32 queries (upper 32 unused), [64,128): delta
+  __shared__ __attribute__((aligned(256))) float lds_s1[128];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int hh = lane >> 5;
+  const int c = lane & 31;
+
+  const int w = blockIdx.x;
+  const int xcd = w & 7, slot = w >> 3;
+  const int per = total_wg >> 3, rem = total_wg & 7;
+  const int vid = xcd * per + (xcd < rem ? xcd : rem) + slot;
+  const int bh = vid / nkb;
+  const int kb = vid - bh * nkb;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+
+  const int64_t Lq = p.Lq, Lk = p.Lk;
+  const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
+  const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
+  const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
+  const E* gp = (const E*)p.dout + (int64_t)b * p.sgb + (int64_t)h * p.sgh;
+  const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
+  const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
+
+  char* q_buf[2] = {reinterpret_cast<char*>(lds_q0), reinterpret_cast<char*>(lds_q1)};
+  char* g_buf[2] = {reinterpret_cast<char*>(lds_g0), reinterpret_cast<char*>(lds_g1)};
+  float* s_buf[2] = {lds_s0, lds_s1};
+
+  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks)
+  const int64_t key = (int64_t)kb * 64 + wave * 32 + c;
+  V8 bk[4], bv[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) {
+    Frag f, g;
+    f.u = make_uint4(0, 0, 0, 0);
+    g.u = make_uint4(0, 0, 0, 0);
+    if (key < Lk) {
+      f.u = *reinterpret_cast<const uint4*>(kp + key * p.skn + ks * 16 + hh * 8);
+      g.u = *reinterpret_cast<const uint4*>(vp + key * p.svn + ks * 16 + hh * 8);
+    }
+    bk[ks] = as_v8<E>(f);
+    bv[ks] = as_v8<E>(g);
+  }
+  f32x16 dkt[2], dvt[2];  // dK^T, dV^T [dt]: lane = key, registers = head_dim
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dkt[dt][r] = 0.f; dvt[dt][r] = 0.f; }
+
+  // query blocks that attend to this key block
+  int n_lists;
+  const int32_t* list = nullptr;
+  if constexpr (DENSE) {
+    n_lists = nqb_all;
+  } else {
+    const int32_t* off = p.kq_off + ((int64_t)b * p.H + h) * (nkb + 1);
+    const int32_t lo = off[kb], hi = off[kb + 1];
+    n_lists = hi - lo;
+    list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo;
+  }
+  auto block_of = [&](int i) -> int64_t {
+    if constexpr (DENSE) return (int64_t)i;
+    else return (int64_t)__builtin_amdgcn_readfirstlane(list[i]);
+  };
+
+  const float sl2 = p.scale * kLog2e;
+  const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
+  const int tr_off = tr_offset(lane);
+
+  // each wave moves half of every half tile (instructions 2*wave, 2*wave+1), wave 0 the lse values, wave 1 delta
+  auto fetch = [&](int64_t qblk, auto hf, int buf) {
+    constexpr int HF = decltype(hf)::value;
+    const int64_t start = qblk * 64;
+    const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
+    dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * HF, last, q_buf[buf], lane, 2 * wave, 2 * wave + 2);
+    dma_rows<E, true>(gp + start * p.sgm, grow, 32 * HF, last, g_buf[buf], lane, 2 * wave, 2 * wave + 2);
+    int r = 32 * HF + c;
+    r = r < last ? r : last;
+    const float* src = (wave == 0 ? lsep : dlp) + start;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, 0x7fffffff, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(s_buf[buf] + 64 * wave), 4, (uint32_t)r * 4u, 0, 0, 0);
+  };
+  auto compute = [&](int64_t qblk, auto hf, int buf) {
+    constexpr int HF = decltype(hf)::value;
+    const int64_t start = qblk * 64;
+    const int nvalid = (int)(Lq - start < 64 ? Lq - start : 64);
+    const bool ragged = nvalid < 64;
+    V8 aq[4], ag[4];
+    read_rows<E, true>(q_buf[buf], c, hh, aq);
+    read_rows<E, true>(g_buf[buf], c, hh, ag);
+    f32x16 s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) s = Mma<E>::mma(aq[ks], bk[ks], s);    // S[q][key]: registers = queries, lane = key
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(ag[ks], bv[ks], dp);  // dP[q][key]
+    V8 pb[2], db[2];  // P and dS as B operands [jj]
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(s_buf[buf] + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(s_buf[buf] + 64 + 4 * hh + 8 * j);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int r = 4 * j + i;
+        float pv = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i] * kLog2e));
+        if (ragged && (32 * HF + 4 * hh + 8 * j + i >= nvalid)) pv = 0.f;
+        pb[r >> 3][r & 7] = (E)pv;
+        db[r >> 3][r & 7] = (E)(pv * (dp[r] - d4[i]) * p.scale);
+      }
+    }
+    V8 gt[2][2], qt[2][2];
+    read_transposed<E>(g_buf[buf], tr_off, gt);
+    read_transposed<E>(q_buf[buf], tr_off, qt);
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++) {
+        dvt[dt] = Mma<E>::mma(gt[jj][dt], pb[jj], dvt[dt]);
+        dkt[dt] = Mma<E>::mma(qt[jj][dt], db[jj], dkt[dt]);
+      }
+  };
+
+  if (n_lists > 0) {
+    int64_t cur = block_of(0);
+    fetch(cur, H0{}, 0);
+    for (int t = 0; t < n_lists; t++) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of half 0 has landed
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of buffer 1 are done
+      __builtin_amdgcn_s_barrier();        // both parts landed; both waves are done with buffer 1
+      fetch(cur, H1{}, 1);
+      compute(cur, H0{}, 0);
+      const bool more = t + 1 < n_lists;
+      const int64_t nxt = more ? block_of(t + 1) : cur;
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();
+      if (more) fetch(nxt, H0{}, 0);
+      compute(cur, H1{}, 1);
+      cur = nxt;
+    }
+  }
+
+  E* dkp = (E*)p.dk + (int64_t)b * p.sdkb + (int64_t)h * p.sdkh;
+  E* dvp = (E*)p.dv + (int64_t)b * p.sdvb + (int64_t)h * p.sdvh;
+  store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
+  store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
+}
+
+}  // namespace bwd
+
+int launch_attn_bwd(const BwdParams& p, int dtype, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  const bool dense = p.idx == nullptr;
+  const int64_t nqb = (p.Lq + 63) / 64, nkb = (p.Lk + 63) / 64;
+  const int64_t nqg = (nqb + 3) / 4;
+  const int64_t total_q = nqg * p.B * p.H, total_k = nkb * p.B * p.H;
+  if (total_q > 0x7fffffffLL || total_k > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "attention backward: grid too large");
+  dim3 gq((unsigned)total_q), bq(256), gk((unsigned)total_k), bk(128);
+#define S3R_BWD_LAUNCH(E)                                                                                                   \
+  do {                                                                                                                      \
+    if (p.dq != nullptr) {                                                                                                  \
+      if (dense) hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, true>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);     \
+      else hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, false>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);          \
+    }                                                                                                                       \
+    if (p.dk != nullptr) {                                                                                                  \
+      if (dense) hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, true>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);   \
+      else hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, false>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);        \
+    }                                                                                                                       \
+  } while (0)
+  if (dtype == S3R_BF16) S3R_BWD_LAUNCH(bf16_t);
+  else S3R_BWD_LAUNCH(f16_t);
+#undef S3R_BWD_LAUNCH
+  return check_launch("attention backward");
+}
+
+int launch_bwd_delta(const void* o, const void* dout, float* delta, int B, int H, int64_t N, int64_t sob, int64_t soh, int64_t son,
+                     int64_t sdb, int64_t sdh, int64_t sdn, int dtype, void* stream) {
+  const int64_t rows = (int64_t)B * H * N;
+  const int64_t blocks = (rows * 8 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd_delta: tensor too large for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)blocks), blk(256);
+  if (dtype == S3R_BF16)
+    hipLaunchKernelGGL(bwd::bwd_delta_kernel<bf16_t>, grid, blk, 0, st, (const bf16_t*)o, (const bf16_t*)dout, delta, H, N, rows, sob, soh, son, sdb, sdh, sdn);
+  else
+    hipLaunchKernelGGL(bwd::bwd_delta_kernel<f16_t>, grid, blk, 0, st, (const f16_t*)o, (const f16_t*)dout, delta, H, N, rows, sob, soh, son, sdb, sdh, sdn);
+  return check_launch("bwd_delta_kernel");
+}
+
+}  // namespace s3r

@@ -30,5 +30,5 @@ def flash_attn_topk_func(q, k, v, topk_val, bias=None, causal=False, softmax_sca
         raise NotImplementedError("flash_attn_topk_func: bias is not supported (the reference kernel ignores it)")
     if causal:
         raise NotImplementedError("flash_attn_topk_func: the causal variant is not provided")
-    o, idx = ops.compressed_attn_topk(q, k, v, topk_val, softmax_scale)
+    o, idx = ops.compressed_attn_topk_autograd(q, k, v, topk_val, softmax_scale)
     return o, idx

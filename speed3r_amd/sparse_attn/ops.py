@@ -280,6 +280,151 @@ def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: to
     return out
 
 
+# ---- backward of the two attention operators --------------------------------------------------------------------
+
+def bwd_supported(q: torch.Tensor, block: int = 64) -> bool:
+    """The backward kernels are built for bf16/fp16, head_dim 64, block 64."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] == 64 and block == 64
+
+
+def key_block_lists(idx: torch.Tensor, n_key_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Key-centric view of the index tensor ``[B,H,Nq_blocks,K]``: for every (b, h) the query-block ids grouped by
+    the key block they list, one entry per occurrence, ascending within a group (stable), and the group offsets
+    ``[B,H,n_key_blocks+1]``; entries < 0 or >= n_key_blocks appear in no group.  Same construction as the
+    reference's count + stable argsort (topk_blocksparse_attention.py:423-554), with torch device routines."""
+    b, h, nqb, kk = idx.shape
+    flat = idx.reshape(b, h, nqb * kk).long()
+    keys = torch.where((flat >= 0) & (flat < n_key_blocks), flat, torch.full_like(flat, n_key_blocks))
+    order = torch.argsort(keys, dim=-1, stable=True)
+    qblk = torch.div(order, kk, rounding_mode="floor").to(torch.int32).contiguous()
+    counts = torch.zeros((b, h, n_key_blocks + 1), dtype=torch.int64, device=idx.device)
+    counts.scatter_add_(-1, keys, torch.ones_like(keys))
+    off = torch.zeros((b, h, n_key_blocks + 1), dtype=torch.int32, device=idx.device)
+    off[..., 1:] = counts[..., :n_key_blocks].cumsum(-1).to(torch.int32)
+    return qblk, off
+
+
+def attn_bwd_delta(o: torch.Tensor, dout: torch.Tensor) -> torch.Tensor:
+    """``delta[b,h,n] = sum_d o * dout`` in fp32."""
+    _need_device(o, dout)
+    o, dout = _last_contig(o), _last_contig(dout)
+    b, h, n, d = o.shape
+    delta = torch.empty((b, h, n), dtype=torch.float32, device=o.device)
+    with torch.cuda.device(o.device):
+        rc = _lib.lib().s3r_attn_bwd_delta(o.data_ptr(), dout.data_ptr(), delta.data_ptr(), b, h, n, d,
+                                           o.stride(0), o.stride(1), o.stride(2),
+                                           dout.stride(0), dout.stride(1), dout.stride(2), _code(o), _stream(o))
+    _lib.check(rc, "s3r_attn_bwd_delta")
+    return delta
+
+
+def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
+             idx: Optional[torch.Tensor] = None, block: int = 64, softmax_scale: Optional[float] = None,
+             need_dq: bool = True, need_dkv: bool = True):
+    """Gradients ``(dq, dk, dv)`` of an attention forward with output ``o`` and log-sum-exp ``lse``:
+    selection attention over the blocks of ``idx`` ([B,H,Nq_blocks,K] int32), or dense attention (``idx=None``)."""
+    _need_device(q, k, v, o, dout, lse)
+    assert bwd_supported(q, block), "attention backward: built for bf16/fp16, head_dim 64, block 64"
+    q, k, v, o, dout = (_last_contig(t) for t in (q, k, v, o, dout))
+    lse = lse.contiguous()
+    b, h, lq, d = q.shape
+    lk = k.shape[2]
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    delta = attn_bwd_delta(o, dout)
+    dq = torch.empty_like(q, memory_format=torch.contiguous_format) if need_dq else None
+    dk = torch.empty_like(k, memory_format=torch.contiguous_format) if need_dkv else None
+    dv = torch.empty_like(v, memory_format=torch.contiguous_format) if need_dkv else None
+    nkb = -(-lk // 64)
+    lists = offs = None
+    kk = 0
+    if idx is not None:
+        idx = _last_contig(idx)
+        assert idx.dtype == torch.int32 and idx.shape[:3] == (b, h, -(-lq // 64))
+        kk = idx.shape[3]
+        if need_dkv:
+            lists, offs = key_block_lists(idx, nkb)
+
+    def st(t):
+        return (t.stride(0), t.stride(1), t.stride(2)) if t is not None else (0, 0, 0)
+
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().s3r_attn_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            idx.data_ptr() if idx is not None else None,
+            lists.data_ptr() if lists is not None else None, offs.data_ptr() if offs is not None else None,
+            lists.shape[-1] if lists is not None else 0,
+            dq.data_ptr() if dq is not None else None, dk.data_ptr() if dk is not None else None,
+            dv.data_ptr() if dv is not None else None,
+            b, h, lq, lk, d, block, kk,
+            *st(q), *st(k), *st(v), *st(dout), *st(dq), *st(dk), *st(dv), *st(idx),
+            scale, _code(q), _stream(q))
+    _lib.check(rc, "s3r_attn_bwd")
+    return dq, dk, dv
+
+
+class _SelectAttnFn(torch.autograd.Function):
+    """Selection attention with gradients (reference TopkBlockSparseAttention, topk_blocksparse_attention.py:1041-1090)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, idx, block, softmax_scale):
+        with torch.no_grad():
+            o, lse = select_attn(q, k, v, idx, block, softmax_scale, return_lse=True)
+        ctx.save_for_backward(q, k, v, o, lse, idx)
+        ctx.block, ctx.scale = block, softmax_scale
+        return o
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, o, lse, idx = ctx.saved_tensors
+        dq, dk, dv = attn_bwd(q, k, v, o, dout, lse, idx, ctx.block, ctx.scale,
+                              need_dq=ctx.needs_input_grad[0], need_dkv=ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
+        return dq, dk, dv, None, None, None
+
+
+class _CompressedAttnFn(torch.autograd.Function):
+    """Compressed attention + top-k with gradients for the attention output (the indices carry none; reference
+    FlashAttnTopkFunc, flash_attention_topk.py:633-665)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, topk, softmax_scale):
+        with torch.no_grad():
+            o, idx, lse = compressed_attn_topk(q, k, v, topk, softmax_scale, return_lse=True)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.scale = softmax_scale
+        if idx is not None:
+            ctx.mark_non_differentiable(idx)
+        return o, idx
+
+    @staticmethod
+    def backward(ctx, dout, _didx):
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = attn_bwd(q, k, v, o, dout, lse, None, 64, ctx.scale,
+                              need_dq=ctx.needs_input_grad[0], need_dkv=ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
+        return dq, dk, dv, None, None
+
+
+def _wants_grad(*ts: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts)
+
+
+def select_attn_autograd(q, k, v, idx, block, softmax_scale=None):
+    """:func:`select_attn`, differentiable in q, k, v where the backward kernels are built."""
+    if not _wants_grad(q, k, v):
+        return select_attn(q, k, v, idx, block, softmax_scale)
+    if not bwd_supported(q, block):
+        raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64, block 64 only")
+    return _SelectAttnFn.apply(q, k, v, idx, block, softmax_scale)
+
+
+def compressed_attn_topk_autograd(q, k, v, topk, softmax_scale=None):
+    """:func:`compressed_attn_topk` (``(o, idx)``), differentiable in q, k, v where the backward kernels are built."""
+    if not _wants_grad(q, k, v):
+        return compressed_attn_topk(q, k, v, topk, softmax_scale)
+    if not bwd_supported(q):
+        raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64 only")
+    return _CompressedAttnFn.apply(q, k, v, topk, softmax_scale)
+
+
 _SIDE_STREAMS = {}
 
 

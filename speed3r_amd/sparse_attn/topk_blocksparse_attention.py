@@ -32,4 +32,4 @@ def topk_blocksparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
     assert topk_idx.shape[0] == batch
     assert topk_idx.shape[1] == nheads
     assert topk_idx.shape[2] == -(-seq_len // block_size)
-    return ops.select_attn(q, k, v, topk_idx, block_size, softmax_scale)
+    return ops.select_attn_autograd(q, k, v, topk_idx, block_size, softmax_scale)

@@ -1,0 +1,122 @@
+"""Parity of the attention backward kernels against the CPU oracle, through the C-ABI (needs an MI355X).
+
+Bar: bf16/fp16 gradients within 2e-2 * max(1, max|reference|) of the oracle's fp32/fp64 gradients on the same
+(already rounded) inputs.  The device forward supplies o and lse, as in training.
+"""
+import pytest
+import torch
+
+import oracle
+import speed3r_amd as s3r
+from speed3r_amd.sparse_attn import ops
+from helpers import max_abs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _randn(shape, seed, dtype, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _close(got, want, what):
+    tol = 2e-2 * max(1.0, float(want.abs().max()))
+    err = max_abs(got, want)
+    assert err <= tol, f"{what}: max abs error {err:.4g} > {tol:.4g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [128, 200, 64, 333])
+def test_delta_is_the_row_dot_product(dtype, n):
+    o, g = _randn((2, 3, n, 64), 1, dtype), _randn((2, 3, n, 64), 2, dtype)
+    got = ops.attn_bwd_delta(o.to(DEV), g.to(DEV))
+    want = (o.float() * g.float()).sum(-1)
+    assert max_abs(got, want) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lq,lk", [(128, 128), (200, 200), (70, 70), (64, 64), (521, 521)])
+def test_dense_backward_matches_oracle(dtype, lq, lk):
+    q, k, v = (_randn((1, 2, l, 64), 10 + i, dtype, 0.5) for i, l in enumerate((lq, lk, lk)))
+    g = _randn((1, 2, lq, 64), 20, dtype)
+    qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, g))
+    o, _, lse = s3r.compressed_attn_topk(qd, kd, vd, None, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse)
+    wq, wk, wv = oracle.compressed_attention_grads_autograd(q, k, v, g)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+
+
+def _rand_idx(b, h, nqb, kk, nkb, seed, lo=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, nkb, (b, h, nqb, kk), generator=g, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,kk", [(512, 4), (1000, 4), (1041, 8), (256, 1), (4100, 16)])
+def test_selection_backward_matches_oracle(dtype, n, kk):
+    b, h = 1, 2
+    nqb = -(-n // 64)
+    q, k, v, g = (_randn((b, h, n, 64), 30 + i, dtype, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb, 40 + n)
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 64, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd)
+    wq, wk, wv = oracle.select_attention_grads_autograd(q, k, v, idx, 64, g)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+
+
+def test_selection_backward_with_skips_duplicates_and_unattended_keys():
+    b, h, n, kk = 1, 2, 640, 4
+    nqb = n // 64
+    q, k, v, g = (_randn((b, h, n, 64), 50 + i, torch.bfloat16, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb - 2, 55, lo=-1)       # -1 entries; key blocks 8, 9 are never attended
+    idx[0, 0, 2] = torch.tensor([3, 3, 3, 1])                   # duplicates
+    idx[0, 1, 4] = -1                                           # a query block that attends nothing
+    idx[0, 1, 5, 0] = nqb + 3                                   # beyond the sequence: skipped
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 64, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd)
+    mult = oracle.block_multiplicity(idx, n, 64)
+    wq, wk, wv, _, _ = oracle.attention_grads_formula(q, k, v, g, mult)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+    assert float(dq[0, 1, 256:320].abs().max()) == 0.0                    # the empty query block
+    assert float(dk[0, :, 512:].abs().max()) == 0.0 and float(dv[0, :, 512:].abs().max()) == 0.0
+
+
+def test_operators_are_differentiable_like_the_reference_ones():
+    b, h, n = 1, 2, 512
+    q, k, v = (_randn((b, h, n, 64), 60 + i, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for i in range(3))
+    g = _randn((b, h, n, 64), 63, torch.bfloat16).to(DEV)
+    idx = _rand_idx(b, h, n // 64, 4, n // 64, 64).to(DEV)
+    o = s3r.topk_blocksparse_attention(q, k, v, idx, 64)
+    o.backward(g)
+    with torch.no_grad():
+        o2, lse = s3r.select_attn(q, k, v, idx, 64, return_lse=True)
+        dq, dk, dv = ops.attn_bwd(q, k, v, o2, g, lse, idx)
+    assert torch.equal(o, o2) and torch.equal(q.grad, dq) and torch.equal(k.grad, dk) and torch.equal(v.grad, dv)
+    # compressed branch: gradients flow through the attention output, the indices carry none
+    qc, kc, vc = (_randn((b, h, 100, 64), 70 + i, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for i in range(3))
+    gc = _randn((b, h, 100, 64), 73, torch.bfloat16)
+    oc, ic = s3r.flash_attn_topk_func(qc, kc, vc, 4)
+    assert not ic.requires_grad and ic.dtype == torch.int32
+    oc.backward(gc.to(DEV))
+    wq, wk, wv = oracle.compressed_attention_grads_autograd(qc.detach().cpu(), kc.detach().cpu(), vc.detach().cpu(), gc)
+    _close(qc.grad, wq, "dq"); _close(kc.grad, wk, "dk"); _close(vc.grad, wv, "dv")
+    # only q wants a gradient: the dk/dv kernel is skipped
+    q2 = q.detach().clone().requires_grad_(True)
+    s3r.topk_blocksparse_attention(q2, k.detach(), v.detach(), idx, 64).backward(g)
+    assert torch.equal(q2.grad, dq)
+
+
+def test_backward_is_linear_in_the_output_gradient_and_sums_over_value_columns():
+    b, h, n, kk = 1, 4, 2048, 8
+    q, k, v, g = (_randn((b, h, n, 64), 80 + i, torch.bfloat16, 0.5 if i < 3 else 1.0).to(DEV) for i in range(4))
+    idx = _rand_idx(b, h, n // 64, kk, n // 64, 85).to(DEV)
+    o, lse = s3r.select_attn(q, k, v, idx, 64, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(q, k, v, o, g, lse, idx)
+    dq2, dk2, dv2 = ops.attn_bwd(q, k, v, o, 2 * g, lse, idx)
+    for a, c2 in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert max_abs(2 * a.float(), c2) <= 2e-2 * max(1.0, float(c2.float().abs().max()))
+    # P sums to one over the attended keys: the column sums of dV equal those of dO (every query block attends something)
+    assert max_abs(dv.float().sum(2), g.float().sum(2)) <= 0.05 * float(g.float().sum(2).abs().max())
