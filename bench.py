@@ -42,6 +42,8 @@ def parse_args():
     ap.add_argument("--no-fuse-merge", action="store_true", help="run selection attention and the gated merge as two kernels")
     ap.add_argument("--overlap", action="store_true",
                     help="run the index kernel on a second stream beside the pooling of v and the compressed attention")
+    ap.add_argument("--backward", action="store_true",
+                    help="time the backward of the two attention operators (one JSON line of its own; not the headline metric)")
     ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "copy"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
@@ -126,6 +128,69 @@ def run_end_to_end(args) -> int:
     return 0
 
 
+def run_backward(args, cfg, qd, kd, vd, block, topk) -> int:
+    """Backward of the selection operator and of the compressed (dense) operator on the forward's tensors: HIP events
+    around delta, the key-centric lists (torch device sort), the dQ kernel and the dK/dV kernel."""
+    import torch
+
+    import speed3r_amd as s3r
+    from speed3r_amd import workloads
+    from speed3r_amd.sparse_attn import ops
+
+    n = cfg.tokens
+    nkb = -(-n // block)
+    with torch.no_grad():
+        qc, kc, vc = s3r.pool_mean(qd, block), s3r.pool_mean(kd, block), s3r.pool_mean(vd, block)
+        oc, idx, lsec = s3r.compressed_attn_topk(qc, kc, vc, topk, return_lse=True)
+        o, lse = s3r.select_attn(qd, kd, vd, idx, block, return_lse=True)
+        g = torch.randn(o.shape, generator=torch.Generator().manual_seed(7)).to(o.dtype).to(o.device)
+        gc = torch.randn(oc.shape, generator=torch.Generator().manual_seed(8)).to(oc.dtype).to(oc.device)
+        names = ["delta", "key_lists", "dq", "dkdv", "compressed_bwd"]
+
+        def step(ev=None):
+            def mark(i):
+                if ev is not None:
+                    ev[i].record()
+            mark(0)
+            delta = ops.attn_bwd_delta(o, g)
+            mark(1)
+            lists = ops.key_block_lists(idx, nkb)
+            mark(2)
+            dq, _, _ = ops.attn_bwd(qd, kd, vd, o, g, lse, idx, block, need_dkv=False, delta=delta)
+            mark(3)
+            _, dk, dv = ops.attn_bwd(qd, kd, vd, o, g, lse, idx, block, need_dq=False, delta=delta, key_lists=lists)
+            mark(4)
+            ops.attn_bwd(qc, kc, vc, oc, gc, lsec)
+            mark(5)
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(evs[i])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms = wall * 1e3 / args.steps
+    kern = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
+    mm = workloads.selection_flops(n, topk) / 2          # one product over the selected (query block, key block) pairs
+    f_dq, f_dkdv = 3 * mm, 4 * mm
+    dom = "dkdv" if kern["dkdv"] >= kern["dq"] else "dq"
+    tfl = (f_dkdv if dom == "dkdv" else f_dq) / (kern[dom] * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "ms/layer backward (selection + compressed attention operators), global sparse attn @%d frames bf16" % cfg.frames,
+        "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{cfg.name} backward: {n} tokens, 16 heads x 64, block {block}, top-k {topk}, B=1"},
+        "kernels_ms": kern,
+        "effective_tflops": (f_dq + f_dkdv + 2.5 * workloads.compressed_flops(n)) / (ms * 1e-3) / 1e12,
+        "roofline": {"kernel": "bwd_dkdv_kernel" if dom == "dkdv" else "bwd_dq_kernel", "bound": "mfma", "achieved": tfl,
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS, "traffic": None},
+    }))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -155,6 +220,9 @@ def main() -> int:
     def step(timeline=None):
         return s3r.sparse_global_attention(qd, kd, vd, gd, block, topk, materialize_scores=mat, fuse_merge=fused,
                                            overlap=overlap, timeline=timeline)
+
+    if args.backward:
+        return run_backward(args, cfg, qd, kd, vd, block, topk)
 
     if args.only:
         with torch.no_grad():

@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 
   // B operands Q and dO (lane = query row, head_dim chunk hh + 2 ks), per-query lse (base 2) and delta
   V8 bq[2][4], bg[2][4];
-  float lse2[2], dlt[2];
+  float lse2[2], dlts[2];  // log-sum-exp in base 2, delta times the softmax scale
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
     const int64_t row = q0 + qt * 32 + c;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       bg[qt][ks] = as_v8<E>(g);
     }
     lse2[qt] = live ? lsep[row] * kLog2e : INFINITY;
-    dlt[qt] = live ? dlp[row] : 0.f;
+    dlts[qt] = live ? dlp[row] * p.scale : 0.f;
   }
   f32x16 dqt[2][2];  // dQ^T accumulators [qt][dt]: lane = query, registers = head_dim
 #pragma unroll
@@ -237,7 +237,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     }
   };
 
-  const float sl2 = p.scale * kLog2e;
+  const float scale = p.scale;
+  const float sl2 = scale * kLog2e;
   const uint32_t krow = (uint32_t)p.skn * (uint32_t)sizeof(E), vrow = (uint32_t)p.svn * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
 
@@ -265,11 +266,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(av[ks], bg[qt][ks], dp);
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float pv = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));
-        if (ragged && (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid)) pv = 0.f;
-        ds[qt][r >> 3][r & 7] = (E)(pv * (dp[r] - dlt[qt]) * p.scale);
+      for (int r = 0; r < 16; r++) st[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));  // P^T
+      if (ragged) {  // keys beyond Lk carry no probability
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) st[r] = 0.f;
       }
+#pragma unroll
+      for (int r = 0; r < 16; r++) ds[qt][r >> 3][r & 7] = (E)(st[r] * fmaf(dp[r], scale, -dlts[qt]));  // scale * P * (dP - delta)
     }
     V8 kt[2][2];
     read_transposed<E>(k_buf[buf], tr_off, kt);
@@ -385,7 +389,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     else return (int64_t)__builtin_amdgcn_readfirstlane(list[i]);
   };
 
-  const float sl2 = p.scale * kLog2e;
+  const float scale = p.scale;
+  const float sl2 = scale * kLog2e;
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
 
@@ -425,11 +430,19 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int r = 4 * j + i;
-        float pv = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i] * kLog2e));
-        if (ragged && (32 * HF + 4 * hh + 8 * j + i >= nvalid)) pv = 0.f;
-        pb[r >> 3][r & 7] = (E)pv;
-        db[r >> 3][r & 7] = (E)(pv * (dp[r] - d4[i]) * p.scale);
+        s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i] * kLog2e));  // P
+        dp[r] = fmaf(dp[r], scale, -d4[i] * scale);                      // scale * (dP - delta)
       }
+    }
+    if (ragged) {  // query rows beyond Lq carry no probability
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) s[r] = 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      pb[r >> 3][r & 7] = (E)s[r];
+      db[r >> 3][r & 7] = (E)(s[r] * dp[r]);
     }
     V8 gt[2][2], qt[2][2];
     read_transposed<E>(g_buf[buf], tr_off, gt);

@@ -320,9 +320,11 @@ def attn_bwd_delta(o: torch.Tensor, dout: torch.Tensor) -> torch.Tensor:
 
 def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
              idx: Optional[torch.Tensor] = None, block: int = 64, softmax_scale: Optional[float] = None,
-             need_dq: bool = True, need_dkv: bool = True):
+             need_dq: bool = True, need_dkv: bool = True, delta: Optional[torch.Tensor] = None,
+             key_lists: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
     """Gradients ``(dq, dk, dv)`` of an attention forward with output ``o`` and log-sum-exp ``lse``:
-    selection attention over the blocks of ``idx`` ([B,H,Nq_blocks,K] int32), or dense attention (``idx=None``)."""
+    selection attention over the blocks of ``idx`` ([B,H,Nq_blocks,K] int32), or dense attention (``idx=None``).
+    ``delta`` (:func:`attn_bwd_delta`) and ``key_lists`` (:func:`key_block_lists`) are computed here unless given."""
     _need_device(q, k, v, o, dout, lse)
     assert bwd_supported(q, block), "attention backward: built for bf16/fp16, head_dim 64, block 64"
     q, k, v, o, dout = (_last_contig(t) for t in (q, k, v, o, dout))
@@ -330,7 +332,8 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
     b, h, lq, d = q.shape
     lk = k.shape[2]
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    delta = attn_bwd_delta(o, dout)
+    if delta is None:
+        delta = attn_bwd_delta(o, dout)
     dq = torch.empty_like(q, memory_format=torch.contiguous_format) if need_dq else None
     dk = torch.empty_like(k, memory_format=torch.contiguous_format) if need_dkv else None
     dv = torch.empty_like(v, memory_format=torch.contiguous_format) if need_dkv else None
@@ -342,7 +345,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
         assert idx.dtype == torch.int32 and idx.shape[:3] == (b, h, -(-lq // 64))
         kk = idx.shape[3]
         if need_dkv:
-            lists, offs = key_block_lists(idx, nkb)
+            lists, offs = key_lists if key_lists is not None else key_block_lists(idx, nkb)
 
     def st(t):
         return (t.stride(0), t.stride(1), t.stride(2)) if t is not None else (0, 0, 0)
