@@ -15,14 +15,14 @@
 //     selected key tiles (or all of them).  Everything is computed transposed, as in the forward kernels:
 //     S^T = K Q^T and dP^T = V dO^T put one QUERY per lane, so lse and delta are per-lane scalars;
 //     dQ^T += K^T dS^T takes K^T fragments from ds_read_b64_tr_b16.  K and V half tiles (32 keys) go global -> LDS
-//     by direct transfers, double buffered (16 KB per wave).  The K half is staged once, in the layout of the
-//     transposed reads; its row reads (A operand of S^T) then take a 2-way bank conflict.
+//     by direct transfers, double buffered (16 KB per wave).  The K half is staged once, in a layout that serves
+//     the transposed reads and the row reads (A operand of S^T) without bank conflicts.
 //   * bwd_dkdv_kernel: one workgroup of two waves per 64-key block, each wave owns 32 keys (one KEY per lane:
 //     S = Q K^T, dP = dO V^T with K, V fragments in registers as B operands) and walks the query blocks that
 //     selected the key block (key-centric lists built by the host from the index tensor, reference :423-554).
-//     Q and dO half tiles (32 queries) and the matching lse / delta values go global -> LDS, shared by the two
-//     waves, double buffered, one barrier per half tile; dV^T += dO^T P and dK^T += Q^T dS read their A operands
-//     transposed from the same buffers.
+//     Q and dO tiles (64 queries) and the matching lse / delta values go global -> LDS, shared by the two waves,
+//     double buffered (the next tile's transfers fly during a whole tile of work), one barrier per tile;
+//     dV^T += dO^T P and dK^T += Q^T dS read their A operands transposed from the same buffers.
 // Query rows beyond Lq have lse = +inf (P = 0), keys beyond Lk are masked (P = 0); rows past the end of a tensor are
 // never read (transfers re-read the last valid row).
 #include "select_common.h"
@@ -65,8 +65,12 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const E* __restrict__ o,
 
 // ---- shared pieces of the two MFMA kernels -----------------------------------------------------------------------
 // Transfer of rows [8*i0*.., ...) of a 32-row half tile: instruction i moves rows 8i .. 8i+7 (16 bytes per lane).
-// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ (((row>>1)&1)<<2) (layout of the transposed reads), else
-// c' ^ (row&7) (layout of conflict-free row reads).  Rows are clamped to `last` (relative to `base`'s row 0).
+// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ tsw(row), tsw = 4*bit1(row) | 2*bit2(row): bit 2 of the chunk
+// spreads the four rows of a transposed read over disjoint bank groups, bit 1 separates rows r and r+4 for the
+// 16-byte row reads, so both kinds of read are conflict free on the same buffer.  Otherwise c' ^ (row&7) (row reads
+// only).  Rows are clamped to `last` (relative to `base`'s row 0).
+__device__ __forceinline__ int tsw(int row) { return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1); }
+
 template <typename E, bool VSW>
 __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int first_row, int last, char* lds_half, int lane, int i_begin, int i_end) {
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
@@ -77,7 +81,7 @@ __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int f
       const int ldsrow = 8 * i + lr;
       int row = first_row + ldsrow;
       row = row < last ? row : last;
-      const int chunk = (lane & 7) ^ (VSW ? (((ldsrow >> 1) & 1) << 2) : (ldsrow & 7));
+      const int chunk = (lane & 7) ^ (VSW ? tsw(ldsrow) : (ldsrow & 7));
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
                                                (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
     }
@@ -87,7 +91,7 @@ __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int f
 // A operand from row reads of a half tile: lane = row c, k-step ks: head_dim chunk 2ks + hh.
 template <typename E, bool VSW>
 __device__ __forceinline__ void read_rows(const char* half, int c, int hh, typename Mma<E>::V8 (&dst)[4]) {
-  const int sw = VSW ? (((c >> 1) & 1) << 2) : (c & 7);
+  const int sw = VSW ? tsw(c) : (c & 7);
 #pragma unroll
   for (int ks = 0; ks < 4; ks++) {
     Frag f;
@@ -117,7 +121,7 @@ __device__ __forceinline__ int tr_offset(int lane) {
   const int hh = lane >> 5;
   const int i16 = lane & 15;
   const int tr_row = 4 * hh + (i16 >> 2);
-  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ tsw(tr_row);
   return tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
 }
 
@@ -319,11 +323,12 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 template <typename E, bool DENSE>
 __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, int nqb_all, int total_wg) {
   typedef typename Mma<E>::V8 V8;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_q0[kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_g0[kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_g1[kHalfBytes];
-  __shared__ __attribute__((aligned(256))) float lds_s0[128];  // [0,64): lse of the half's 32 queries (upper 32 unused), [64,128): delta
+  constexpr int kTileBytes = 2 * kHalfBytes;  // a 64-row query tile
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_q0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_g0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_g1[kTileBytes];
+  __shared__ __attribute__((aligned(256))) float lds_s0[128];  // [0,64): lse of the tile's 64 queries, [64,128): delta
   __shared__ __attribute__((aligned(256))) float lds_s1[128];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -347,10 +352,6 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const E* gp = (const E*)p.dout + (int64_t)b * p.sgb + (int64_t)h * p.sgh;
   const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
   const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
-
-  char* q_buf[2] = {reinterpret_cast<char*>(lds_q0), reinterpret_cast<char*>(lds_q1)};
-  char* g_buf[2] = {reinterpret_cast<char*>(lds_g0), reinterpret_cast<char*>(lds_g1)};
-  float* s_buf[2] = {lds_s0, lds_s1};
 
   // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks)
   const int64_t key = (int64_t)kb * 64 + wave * 32 + c;
@@ -394,27 +395,44 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
 
-  // each wave moves half of every half tile (instructions 2*wave, 2*wave+1), wave 0 the lse values, wave 1 delta
-  auto fetch = [&](int64_t qblk, auto hf, int buf) {
-    constexpr int HF = decltype(hf)::value;
+  float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight
+  float* staged_to = nullptr;  // where it goes in LDS
+  // One query tile (64 rows of Q and dO, 64 lse and delta values) -> buffer BUF; each wave moves half of every
+  // operand (instructions 2*wave, 2*wave+1 of both 32-row halves), wave 0 the lse values, wave 1 delta.
+  auto fetch = [&](int64_t qblk, auto bufc) {
+    constexpr int BUF = decltype(bufc)::value;
+    char* qb = reinterpret_cast<char*>(BUF == 0 ? lds_q0 : lds_q1);
+    char* gb = reinterpret_cast<char*>(BUF == 0 ? lds_g0 : lds_g1);
+    float* sb = BUF == 0 ? lds_s0 : lds_s1;
     const int64_t start = qblk * 64;
     const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
-    dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * HF, last, q_buf[buf], lane, 2 * wave, 2 * wave + 2);
-    dma_rows<E, true>(gp + start * p.sgm, grow, 32 * HF, last, g_buf[buf], lane, 2 * wave, 2 * wave + 2);
-    int r = 32 * HF + c;
-    r = r < last ? r : last;
-    const float* src = (wave == 0 ? lsep : dlp) + start;
-    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, 0x7fffffff, 0x00020000);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(s_buf[buf] + 64 * wave), 4, (uint32_t)r * 4u, 0, 0, 0);
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+      dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * hf, last, qb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+      dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+    }
+    // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
+    // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
+    const int r = lane < last ? lane : last;
+    staged = ((wave == 0 ? lsep : dlp) + start)[r] * (wave == 0 ? kLog2e : scale);
+    staged_to = sb + 64 * wave + lane;
   };
-  auto compute = [&](int64_t qblk, auto hf, int buf) {
+  auto publish = [&]() {
+    if (staged_to != nullptr) *staged_to = staged;
+    staged_to = nullptr;
+  };
+  auto compute = [&](int64_t qblk, auto bufc, auto hf) {
+    constexpr int BUF = decltype(bufc)::value;
     constexpr int HF = decltype(hf)::value;
+    const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
+    const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
+    const float* sb = (BUF == 0 ? lds_s0 : lds_s1) + 32 * HF;
     const int64_t start = qblk * 64;
     const int nvalid = (int)(Lq - start < 64 ? Lq - start : 64);
     const bool ragged = nvalid < 64;
     V8 aq[4], ag[4];
-    read_rows<E, true>(q_buf[buf], c, hh, aq);
-    read_rows<E, true>(g_buf[buf], c, hh, ag);
+    read_rows<E, true>(qb, c, hh, aq);
+    read_rows<E, true>(gb, c, hh, ag);
     f32x16 s, dp;
 #pragma unroll
     for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
@@ -425,13 +443,13 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     V8 pb[2], db[2];  // P and dS as B operands [jj]
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(s_buf[buf] + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(s_buf[buf] + 64 + 4 * hh + 8 * j);
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sb + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sb + 64 + 4 * hh + 8 * j);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int r = 4 * j + i;
-        s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i] * kLog2e));  // P
-        dp[r] = fmaf(dp[r], scale, -d4[i] * scale);                      // scale * (dP - delta)
+        s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i]));  // P (l4: lse in base 2)
+        dp[r] = fmaf(dp[r], scale, -d4[i]);                     // scale * (dP - delta) (d4: delta * scale)
       }
     }
     if (ragged) {  // query rows beyond Lq carry no probability
@@ -445,8 +463,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       db[r >> 3][r & 7] = (E)(s[r] * dp[r]);
     }
     V8 gt[2][2], qt[2][2];
-    read_transposed<E>(g_buf[buf], tr_off, gt);
-    read_transposed<E>(q_buf[buf], tr_off, qt);
+    read_transposed<E>(gb, tr_off, gt);
+    read_transposed<E>(qb, tr_off, qt);
 #pragma unroll
     for (int jj = 0; jj < 2; jj++)
 #pragma unroll
@@ -455,24 +473,32 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         dkt[dt] = Mma<E>::mma(qt[jj][dt], db[jj], dkt[dt]);
       }
   };
+  // this wave's part of the tile has landed, its reads of the other buffer are done; after the barrier both hold
+  // for both waves
+  auto sync = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    publish();
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+  };
 
   if (n_lists > 0) {
     int64_t cur = block_of(0);
-    fetch(cur, H0{}, 0);
-    for (int t = 0; t < n_lists; t++) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of half 0 has landed
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of buffer 1 are done
-      __builtin_amdgcn_s_barrier();        // both parts landed; both waves are done with buffer 1
-      fetch(cur, H1{}, 1);
-      compute(cur, H0{}, 0);
-      const bool more = t + 1 < n_lists;
-      const int64_t nxt = more ? block_of(t + 1) : cur;
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      __builtin_amdgcn_s_barrier();
-      if (more) fetch(nxt, H0{}, 0);
-      compute(cur, H1{}, 1);
-      cur = nxt;
+    fetch(cur, H0{});
+    for (int t = 0; t < n_lists; t += 2) {
+      sync();
+      const bool more1 = t + 1 < n_lists;
+      const int64_t nxt1 = more1 ? block_of(t + 1) : cur;
+      if (more1) fetch(nxt1, H1{});
+      compute(cur, H0{}, H0{});
+      compute(cur, H0{}, H1{});
+      if (!more1) break;
+      sync();
+      const bool more2 = t + 2 < n_lists;
+      cur = more2 ? block_of(t + 2) : nxt1;
+      if (more2) fetch(cur, H0{});
+      compute(nxt1, H1{}, H0{});
+      compute(nxt1, H1{}, H1{});
     }
   }
 
