@@ -8,7 +8,9 @@ Differences, all on the host side of the operator boundary:
 * q, k, v are handed to the kernels as strided views of the packed projection (no ``.contiguous()`` copies),
   pooling reads the packed projection directly, and the gated merge runs in the selection kernel's epilogue
   (or in its own kernel where that is not built), writing ``[B, N, C]`` for ``proj``;
-* forward only: run it under ``torch.no_grad()``;
+* when a gradient is wanted (grad mode on and the input or a parameter requires grad) the layer runs as a
+  differentiable composition instead: the two attention operators with their backward kernels (bf16/fp16,
+  head_dim 64, block 64), pooling, norm/RoPE and merge as torch expressions;
 * ``N`` need not be a multiple of the block: the last block pools its valid tokens, its keys beyond ``N`` are
   masked and its query rows beyond ``N`` do not exist (the reference raises for such ``N``);
 * the top-k count, 32 in the reference, is a constructor argument.
@@ -83,7 +85,50 @@ class SparseFlashAttentionRope(nn.Module):
         t = norm(t).to(t.dtype)
         return self.rope(t, pos) if pos is not None else t
 
+    def _forward_with_grad(self, x: Tensor, xpos: Optional[Tensor]) -> Tensor:
+        """The same layer as a differentiable composition (training): the two attention operators carry their own
+        backward kernels; pooling, qk-norm/RoPE and the gated merge run as the torch expressions of the reference
+        (sparse_attention.py:97-110,120-136), whose gradients autograd provides."""
+        b, n, c = x.shape
+        h = self.num_heads
+        d = c // h
+        block = self.block_size ** 2
+        nc = -(-n // block)
+        qkv = self.qkv(x)
+        gate = self.gate(x).view(b, n, h, 2).permute(0, 2, 1, 3)              # [B, H, N, 2]
+        q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)    # each [B, H, N, D]
+
+        def pool(t):  # block means; a ragged tail block averages its valid tokens
+            pad = nc * block - n
+            tf = torch.nn.functional.pad(t, (0, 0, 0, pad)) if pad else t
+            sums = tf.reshape(b, h, nc, block, d).float().sum(dim=3)
+            counts = torch.full((nc, 1), float(block), device=t.device)
+            if pad:
+                counts[-1] = float(block - pad)
+            return (sums / counts).to(t.dtype)
+
+        def norm_rope(t, norm, pos):
+            t = norm(t).to(t.dtype)
+            return self.rope(t, pos) if pos is not None else t
+
+        use_pos = xpos is not None and self.rope is not None
+        pos_c = block_positions(xpos, block) if use_pos else None
+        q_c, k_c, v_c = pool(q), pool(k), pool(v)
+        q_c, k_c = norm_rope(q_c, self.q_norm, pos_c), norm_rope(k_c, self.k_norm, pos_c)
+        o_c, idx = flash_attn_topk_func(q_c, k_c, v_c, self.topk)
+        if self.keep_topk_idx:
+            self.last_topk_idx = idx
+        pos = xpos if use_pos else None
+        q, k = norm_rope(q, self.q_norm, pos), norm_rope(k, self.k_norm, pos)
+        o_s = ops.select_attn_autograd(q, k, v, idx, block)
+        blk = torch.arange(n, device=x.device) // block
+        out = gate[..., 0:1] * o_c[:, :, blk] + gate[..., 1:2] * o_s           # [B, H, N, D]
+        out = out.permute(0, 2, 1, 3).reshape(b, n, c)
+        return self.proj_drop(self.proj(out))
+
     def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            return self._forward_with_grad(x, xpos)
         b, n, c = x.shape
         h = self.num_heads
         d = c // h

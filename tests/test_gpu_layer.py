@@ -65,11 +65,13 @@ def test_layer_without_norm_and_positions():
     assert max_abs(got, ref["out"].float()) <= 4e-2
 
 
-def test_layer_is_forward_only():
-    m = _make(128, 2, 8, 2, torch.bfloat16, seed=7).to(DEV)
+def test_layer_refuses_gradients_where_no_backward_kernel_is_built():
+    m = _make(128, 2, 4, 2, torch.bfloat16, seed=7).to(DEV)      # block 16: the backward kernels are built for block 64
     x = torch.randn((1, 128, 128), device=DEV, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError):
         m(x)                      # parameters require grad and grad mode is on
+    with torch.no_grad():
+        assert m(x).shape == x.shape
 
 
 # ------------------------------------------------------------------------------------ fused qk-norm + RoPE kernel
@@ -104,3 +106,42 @@ def test_norm_rope_kernel_matches_the_torch_modules(dtype, with_norm, with_pos):
         assert torch.equal(got, want)                                              # no reduction involved: bit-identical
     elif dtype != torch.float32:
         assert (got == want).float().mean().item() >= 0.97
+
+
+@pytest.mark.parametrize("n", [320, 200])
+def test_layer_gradients_match_autograd_through_the_oracle(n):
+    b, dim, heads, block_size, topk = 1, 128, 2, 8, 2
+    m = _make(dim, heads, block_size, topk, torch.bfloat16, seed=40 + n)
+    g = torch.Generator().manual_seed(41 + n)
+    x = torch.randn((b, n, dim), generator=g).to(torch.bfloat16)
+    gout = torch.randn((b, n, dim), generator=g).to(torch.bfloat16)
+    side = 24
+    xpos = torch.stack((torch.arange(n) // side, torch.arange(n) % side), dim=-1)[None].expand(b, n, 2).contiguous()
+    m.to(DEV).train()
+    m.keep_topk_idx = True
+    xd = x.to(DEV).requires_grad_(True)
+    out = m(xd, xpos=xpos.to(DEV))
+    with torch.no_grad():
+        m.eval()
+        ref_fwd = m(x.to(DEV), xpos=xpos.to(DEV))        # the inference path (fused kernels) on the same weights
+        m.train()
+    assert max_abs(out.detach(), ref_fwd) <= 4e-2
+    out.backward(gout.to(DEV))
+    idx = m.last_topk_idx.cpu()
+    got = {k: p.grad.detach().float().cpu() for k, p in m.named_parameters() if p.grad is not None}
+    got["x"] = xd.grad.detach().float().cpu()
+    # the oracle in fp32 on the same (bf16-rounded) parameters and the module's block choice
+    m.cpu()
+    params = {k: v.detach().float().requires_grad_(True) for k, v in m.state_dict().items()}
+    xr = x.float().requires_grad_(True)
+    ref = oracle.sparse_layer(xr, params["qkv.weight"], params.get("qkv.bias"), params["gate.0.weight"], params["gate.0.bias"],
+                              params["proj.weight"], params.get("proj.bias"), heads, block_size ** 2, topk, xpos=xpos,
+                              qn_w=params.get("q_norm.weight"), qn_b=params.get("q_norm.bias"),
+                              kn_w=params.get("k_norm.weight"), kn_b=params.get("k_norm.bias"), idx_override=idx)
+    ref["out"].backward(gout.float())
+    want = {k: v.grad for k, v in params.items() if v.grad is not None}
+    want["x"] = xr.grad
+    assert set(want) == set(got), (sorted(want), sorted(got))
+    for k in want:
+        tol = 5e-2 * max(1.0, float(want[k].abs().max()))
+        assert max_abs(got[k], want[k]) <= tol, (k, max_abs(got[k], want[k]), tol)
