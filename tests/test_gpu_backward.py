@@ -120,3 +120,46 @@ def test_backward_is_linear_in_the_output_gradient_and_sums_over_value_columns()
         assert max_abs(2 * a.float(), c2) <= 2e-2 * max(1.0, float(c2.float().abs().max()))
     # P sums to one over the attended keys: the column sums of dV equal those of dO (every query block attends something)
     assert max_abs(dv.float().sum(2), g.float().sum(2)) <= 0.05 * float(g.float().sum(2).abs().max())
+
+
+def test_backward_at_full_size_on_sampled_blocks():
+    # 266 496 tokens, 16 heads, top-k 16 (the headline shape): gradients of sampled query blocks (dq) and key blocks
+    # (dk, dv) against an fp32 restatement of the formulas on the device
+    from speed3r_amd import workloads
+
+    cfg, q, k, v, _ = workloads.make_config("cfg3")
+    n, nb, kk = cfg.tokens, cfg.tokens // 64, cfg.topk
+    q, k, v = (t.to(DEV) for t in (q, k, v))
+    qc, kc, vc = (s3r.pool_mean(t, 64) for t in (q, k, v))
+    _, idx = s3r.compressed_attn_topk(qc, kc, vc, kk)
+    o, lse = s3r.select_attn(q, k, v, idx, 64, return_lse=True)
+    g = torch.randn(o.shape, generator=torch.Generator().manual_seed(90)).to(torch.bfloat16).to(DEV)
+    dq, dk, dv = ops.attn_bwd(q, k, v, o, g, lse, idx)
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
+    delta = (o.float() * g.float()).sum(-1)                                           # [1, 16, n]
+    lists, off = ops.key_block_lists(idx, nb)
+    gen = torch.Generator().manual_seed(91)
+    ar = torch.arange(64, device=DEV)
+    for m in torch.randint(0, nb, (6,), generator=gen).tolist():                      # query blocks
+        rows = slice(64 * m, 64 * m + 64)
+        tok = (idx[0, :, m].long()[:, :, None] * 64 + ar).reshape(16, kk * 64)        # [16 heads, K*64] key tokens
+        kg = k[0].gather(1, tok[:, :, None].expand(16, kk * 64, 64)).float()
+        vg = v[0].gather(1, tok[:, :, None].expand(16, kk * 64, 64)).float()
+        p = torch.exp(q[0, :, rows].float() @ kg.transpose(1, 2) / 8.0 - lse[0, :, rows, None])
+        ds = p * (g[0, :, rows].float() @ vg.transpose(1, 2) - delta[0, :, rows, None]) / 8.0
+        want = ds @ kg
+        assert max_abs(dq[0, :, rows], want) <= 2e-2 * max(1.0, float(want.abs().max()))
+    for j in torch.randint(0, nb, (6,), generator=gen).tolist():                      # key blocks
+        keys = slice(64 * j, 64 * j + 64)
+        for h in (0, 7, 15):
+            lo, hi = int(off[0, h, j]), int(off[0, h, j + 1])
+            want_dk = torch.zeros((64, 64), device=DEV)
+            want_dv = torch.zeros((64, 64), device=DEV)
+            if hi > lo:
+                qtok = (lists[0, h, lo:hi].long()[:, None] * 64 + ar).reshape(-1)     # query tokens attending block j
+                qf, gf = q[0, h, qtok].float(), g[0, h, qtok].float()
+                p = torch.exp(qf @ k[0, h, keys].float().T / 8.0 - lse[0, h, qtok, None])
+                ds = p * (gf @ v[0, h, keys].float().T - delta[0, h, qtok, None]) / 8.0
+                want_dk, want_dv = ds.T @ qf, p.T @ gf
+            assert max_abs(dk[0, h, keys], want_dk) <= 2e-2 * max(1.0, float(want_dk.abs().max()))
+            assert max_abs(dv[0, h, keys], want_dv) <= 2e-2 * max(1.0, float(want_dv.abs().max()))
