@@ -421,26 +421,29 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     if (staged_to != nullptr) *staged_to = staged;
     staged_to = nullptr;
   };
-  auto compute = [&](int64_t qblk, auto bufc, auto hf) {
+  // One tile in three stages per 32-query half, issued so that the matrix products of one half run under the
+  // vector work of the other: A = row reads + S, dP; B = P and dS from the per-query scalars; C = transposed reads +
+  // dV^T, dK^T.
+  auto stage_a = [&](auto bufc, auto hf, f32x16& s, f32x16& dp) {
     constexpr int BUF = decltype(bufc)::value;
     constexpr int HF = decltype(hf)::value;
     const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
     const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
-    const float* sb = (BUF == 0 ? lds_s0 : lds_s1) + 32 * HF;
-    const int64_t start = qblk * 64;
-    const int nvalid = (int)(Lq - start < 64 ? Lq - start : 64);
-    const bool ragged = nvalid < 64;
     V8 aq[4], ag[4];
     read_rows<E, true>(qb, c, hh, aq);
     read_rows<E, true>(gb, c, hh, ag);
-    f32x16 s, dp;
 #pragma unroll
     for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) s = Mma<E>::mma(aq[ks], bk[ks], s);    // S[q][key]: registers = queries, lane = key
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(ag[ks], bv[ks], dp);  // dP[q][key]
-    V8 pb[2], db[2];  // P and dS as B operands [jj]
+  };
+  auto stage_b = [&](int64_t qblk, auto bufc, auto hf, f32x16& s, f32x16& dp, V8 (&pb)[2], V8 (&db)[2]) {
+    constexpr int BUF = decltype(bufc)::value;
+    constexpr int HF = decltype(hf)::value;
+    const float* sb = (BUF == 0 ? lds_s0 : lds_s1) + 32 * HF;
+    const int nvalid = (int)(Lq - qblk * 64 < 64 ? Lq - qblk * 64 : 64);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(sb + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
@@ -452,7 +455,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         dp[r] = fmaf(dp[r], scale, -d4[i]);                     // scale * (dP - delta) (d4: delta * scale)
       }
     }
-    if (ragged) {  // query rows beyond Lq carry no probability
+    if (nvalid < 64) {  // query rows beyond Lq carry no probability
 #pragma unroll
       for (int r = 0; r < 16; r++)
         if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) s[r] = 0.f;
@@ -462,6 +465,12 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       pb[r >> 3][r & 7] = (E)s[r];
       db[r >> 3][r & 7] = (E)(s[r] * dp[r]);
     }
+  };
+  auto stage_c = [&](auto bufc, auto hf, const V8 (&pb)[2], const V8 (&db)[2]) {
+    constexpr int BUF = decltype(bufc)::value;
+    constexpr int HF = decltype(hf)::value;
+    const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
+    const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
     V8 gt[2][2], qt[2][2];
     read_transposed<E>(gb, tr_off, gt);
     read_transposed<E>(qb, tr_off, qt);
@@ -472,6 +481,16 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         dvt[dt] = Mma<E>::mma(gt[jj][dt], pb[jj], dvt[dt]);
         dkt[dt] = Mma<E>::mma(qt[jj][dt], db[jj], dkt[dt]);
       }
+  };
+  auto compute_tile = [&](int64_t qblk, auto bufc) {
+    f32x16 s0, dp0, s1, dp1;
+    V8 pb0[2], db0[2], pb1[2], db1[2];
+    stage_a(bufc, H0{}, s0, dp0);
+    stage_a(bufc, H1{}, s1, dp1);
+    stage_b(qblk, bufc, H0{}, s0, dp0, pb0, db0);
+    stage_c(bufc, H0{}, pb0, db0);
+    stage_b(qblk, bufc, H1{}, s1, dp1, pb1, db1);
+    stage_c(bufc, H1{}, pb1, db1);
   };
   // this wave's part of the tile has landed, its reads of the other buffer are done; after the barrier both hold
   // for both waves
@@ -490,15 +509,13 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       const bool more1 = t + 1 < n_lists;
       const int64_t nxt1 = more1 ? block_of(t + 1) : cur;
       if (more1) fetch(nxt1, H1{});
-      compute(cur, H0{}, H0{});
-      compute(cur, H0{}, H1{});
+      compute_tile(cur, H0{});
       if (!more1) break;
       sync();
       const bool more2 = t + 2 < n_lists;
       cur = more2 ? block_of(t + 2) : nxt1;
       if (more2) fetch(cur, H0{});
-      compute(nxt1, H1{}, H0{});
-      compute(nxt1, H1{}, H1{});
+      compute_tile(nxt1, H1{});
     }
   }
 
