@@ -116,6 +116,11 @@ static int select_attn_impl(const char* who, const void* q, const void* k, const
     return launch_select_pipe(p, dtype, stream);
   }
   if (mfma_ok) return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
+  // 16-token blocks (the reference layer's own setting): MFMA kernel that pairs query blocks
+  const bool b16_ok = dtype != S3R_F32 && D == 64 && block == 16 && K <= 64 && softmax_scale > 0.f &&
+                      skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
+                      vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, son);
+  if (b16_ok) return launch_select_b16(p, dtype, stream);
   return launch_attn_simple(p, dtype, /*select=*/true, stream);
 }
 

@@ -1,0 +1,275 @@
+// Selection-branch attention for 16-token blocks on the gfx950 matrix cores (bf16 / fp16 I/O, head_dim 64):
+// the reference layer's own setting, block_size**2 = 16 with 32 blocks per query block
+// (pi3/models/layers/sparse_attention.py:73,98,125; kernel topk_blocksparse_attention.py:35-128).
+//
+// One wavefront owns four consecutive query blocks (64 queries) of one head; four independent waves per workgroup.
+// The 32x32x16 MFMA wants 32 keys and 32 queries per tile, a query block has only 16 of each per list entry, so a
+// tile pairs TWO query blocks with ONE list entry of each: rows 0-15 of the key half tile hold the block the first
+// query block lists at position i, rows 16-31 the block the second one lists at position i.  S^T = K Q^T then has
+// two useful 16x16 quadrants (first block's keys x first block's queries, second x second); the other two are
+// masked to probability zero.  Half of the matrix work is thrown away, which is affordable: this shape is bound by
+// the texture path (a 2 KB key block serves 16 queries, a quarter of the reuse of the 64-token case), not by MFMA.
+// Everything else follows the 64-token kernels: one query per lane (S^T accumulator), P rounded to the I/O dtype,
+// O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16, K/V half tiles by direct transfers with explicit waits,
+// double buffered (the two query-block pairs of the wave alternate, so pair 1's tiles fly while pair 0 computes).
+// The softmax is online (running maximum per query, accumulators rescaled only when some maximum moved).
+// Entries < 0 or starting at or beyond N are skipped, keys beyond N in the ragged last block are masked, a query
+// block with no valid entry gives zeros; up to 64 entries per query block.
+#include "select_common.h"
+#include "attn_params.h"
+
+namespace s3r {
+namespace b16 {
+using namespace sel;
+
+constexpr int kHalfBytes = 32 * 128;
+constexpr float kLog2e = 1.4426950408889634f;
+typedef std::integral_constant<int, 0> H0;
+typedef std::integral_constant<int, 1> H1;
+
+template <typename E>
+__global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nqb, int ngrp, int nwg_per_bh, int total_wg) {
+  typedef typename Mma<E>::V8 V8;
+  typedef typename Mma<E>::V2 V2;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[4 * kHalfBytes];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int hh = lane >> 5;
+  const int c = lane & 31;
+
+  const int w = blockIdx.x;  // XCD-aware: each XCD walks a contiguous range of query groups of one head
+  const int xcd = w & 7, slot = w >> 3;
+  const int per = total_wg >> 3, rem = total_wg & 7;
+  const int vid = xcd * per + (xcd < rem ? xcd : rem) + slot;
+  const int bh = vid / nwg_per_bh;
+  const int wg = vid - bh * nwg_per_bh;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+  const int grp = wg * 4 + wave;  // group of four query blocks = 64 queries
+  if (grp >= ngrp) return;
+
+  const int64_t N = p.Lq;
+  const int64_t q0 = (int64_t)grp * 64;
+  const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
+  const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
+  const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
+  E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
+
+  char* k_buf[2] = {reinterpret_cast<char*>(lds_k0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_k1) + wave * kHalfBytes};
+  char* v_buf[2] = {reinterpret_cast<char*>(lds_v0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_v1) + wave * kHalfBytes};
+
+  // B operand Q: lane = query row, head_dim chunk hh + 2 ks
+  V8 bq[2][4];
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++) {
+    const int64_t row = q0 + qt * 32 + c;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      Frag f;
+      f.u = make_uint4(0, 0, 0, 0);
+      if (row < N) f.u = *reinterpret_cast<const uint4*>(qp + row * p.sqm + ks * 16 + hh * 8);
+      bq[qt][ks] = as_v8<E>(f);
+    }
+  }
+  // the four index rows of the group, one entry per lane
+  int32_t my_idx[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int qb = grp * 4 + j;
+    my_idx[j] = -1;
+    if (qb < nqb && lane < p.K) my_idx[j] = p.idx[(int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim + lane];
+    if (my_idx[j] < 0 || (int64_t)my_idx[j] * 16 >= N) my_idx[j] = -1;
+  }
+
+  f32x16 ot[2][2];  // O^T [dt][qt]
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) ot[dt][qt][r] = 0.f;
+  float m_i[2] = {-INFINITY, -INFINITY}, l_i[2] = {0.f, 0.f};
+  const float sl2 = p.scale * kLog2e;
+  const uint32_t krow = (uint32_t)p.skn * (uint32_t)sizeof(E), vrow = (uint32_t)p.svn * (uint32_t)sizeof(E);
+
+  // per-lane pieces of the transfers and reads
+  const int lr = lane >> 3;
+  const int i16 = lane & 15;
+  const int tr_row = 4 * hh + (i16 >> 2);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
+  const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
+  const int kr_off = c * 128 + ((hh ^ (c & 7)) << 4);
+
+  // Unit (i, QT): list position i of query blocks 2 QT and 2 QT + 1.  blk[0], blk[1]: their key blocks (-1: skip).
+  auto entry = [&](int i, auto qt_tag, int32_t (&blk)[2]) {
+    constexpr int QT = decltype(qt_tag)::value;
+    blk[0] = __builtin_amdgcn_readlane(my_idx[2 * QT], i);
+    blk[1] = __builtin_amdgcn_readlane(my_idx[2 * QT + 1], i);
+  };
+  auto fetch = [&](int i, auto qt_tag) {  // the unit's K and V half tiles -> buffers QT (skipped blocks re-read block 0)
+    constexpr int QT = decltype(qt_tag)::value;
+    int32_t blk[2];
+    entry(i, qt_tag, blk);
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      const int64_t start = (int64_t)(blk[s] < 0 ? 0 : blk[s]) * 16;
+      const int last = (int)((N - start < 16 ? N - start : 16) - 1);
+      const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + start * p.svn), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const int ldsrow = 16 * s + 8 * t + lr;   // row of the 32-row half tile
+        int row = 8 * t + lr;                     // row of the 16-token block
+        row = row < last ? row : last;
+        const uint32_t kc = (uint32_t)(((lane & 7) ^ (ldsrow & 7)) * 16);
+        const uint32_t vc = (uint32_t)(((lane & 7) ^ (((ldsrow >> 1) & 1) << 2)) * 16);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(k_buf[QT] + (2 * s + t) * 1024), 16,
+                                                 (uint32_t)row * krow + kc, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(v_buf[QT] + (2 * s + t) * 1024), 16,
+                                                 (uint32_t)row * vrow + vc, 0, 0, 0);
+      }
+    }
+  };
+  auto compute = [&](int i, auto qt_tag) {
+    constexpr int QT = decltype(qt_tag)::value;
+    int32_t blk[2];
+    entry(i, qt_tag, blk);
+    // this lane's query belongs to block `mine` of the pair; only that block's 16 keys count for it
+    const int mine = c >> 4;
+    const int32_t myblk = mine == 0 ? blk[0] : blk[1];
+    const int nkeys = myblk < 0 ? 0 : (int)(N - (int64_t)myblk * 16 < 16 ? N - (int64_t)myblk * 16 : 16);
+    V8 ak[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      Frag f;
+      f.u = *reinterpret_cast<const uint4*>(k_buf[QT] + (kr_off ^ (ks << 5)));
+      ak[ks] = as_v8<E>(f);
+    }
+    f32x16 st;
+#pragma unroll
+    for (int r = 0; r < 16; r++) st[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) st = Mma<E>::mma(ak[ks], bq[QT][ks], st);
+    // register r holds key row 4hh + 8(r/4) + r%4 of the half tile: rows 0-15 (r < 8) are block 0's keys, 16-31 block 1's
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int krow_in_blk = 4 * hh + 8 * ((r >> 2) & 1) + (r & 3);
+      const bool ok = ((r >> 3) == mine) && (krow_in_blk < nkeys);
+      st[r] = ok ? st[r] * sl2 : -INFINITY;
+      mx = fmaxf(mx, st[r]);
+    }
+    mx = xh_max(mx);
+    const float m_new = fmaxf(m_i[QT], mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing valid so far: every probability is exp2(-inf) = 0
+    const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - m_use);  // 0 while m_i is -inf
+    if (__any(m_new != m_i[QT])) {
+      l_i[QT] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
+    }
+    m_i[QT] = m_new;
+    V8 pf[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        V2 pk;
+        pk[0] = (E)__builtin_amdgcn_exp2f(st[8 * jj + e] - m_use);
+        pk[1] = (E)__builtin_amdgcn_exp2f(st[8 * jj + e + 1] - m_use);
+        pf[jj][e] = pk[0];
+        pf[jj][e + 1] = pk[1];
+        l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
+      }
+    V8 vfr[2][2];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++) {
+        const char* a0 = v_buf[QT] + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+        Frag f;
+        f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+        f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+        vfr[jj][dt] = as_v8<E>(f);
+      }
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[jj], ot[dt][QT]);
+  };
+
+  const int nsteps = p.K;
+  if (nsteps > 0) {
+    fetch(0, H0{});
+    for (int i = 0; i < nsteps; i++) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 1 (previous step) are done
+      fetch(i, H1{});
+      __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 0) has landed
+      compute(i, H0{});
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 0 are done
+      if (i + 1 < nsteps) {
+        fetch(i + 1, H0{});
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 1) has landed
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
+      compute(i, H1{});
+    }
+  }
+
+  // output: as in the 64-token kernels (one exchange with lane ^ 32 per packed word, 16-byte stores)
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++) {
+    const float l = xh_sum(l_i[qt]);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const int64_t row = q0 + qt * 32 + c;
+    const bool live = row < N;
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int gp = 0; gp < 2; gp++) {
+        union { E e[8]; uint32_t w[4]; uint4 u; } pc;
+        union { E e[2]; uint32_t w; } t;
+#pragma unroll
+        for (int wi = 0; wi < 2; wi++) {
+          t.e[0] = (E)(ot[dt][qt][8 * gp + 2 * wi] * inv);
+          t.e[1] = (E)(ot[dt][qt][8 * gp + 2 * wi + 1] * inv);
+          const uint32_t a = t.w;
+          t.e[0] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi] * inv);
+          t.e[1] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi + 1] * inv);
+          const uint32_t bw = t.w;
+          const auto r = __builtin_amdgcn_permlane32_swap(a, bw, false, false);
+          pc.w[wi] = r[0];
+          pc.w[2 + wi] = r[1];
+        }
+        if (live) *reinterpret_cast<uint4*>(op + row * p.som + dt * 32 + 8 * (2 * gp + hh)) = pc.u;
+      }
+    if (live && p.lse != nullptr && hh == 0)
+      p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+  }
+}
+
+}  // namespace b16
+
+int launch_select_b16(const AttnParams& p, int dtype, void* stream) {
+  const int64_t nqb = (p.Lq + 15) / 16;
+  const int64_t ngrp = (nqb + 3) / 4;
+  const int64_t nwg = (ngrp + 3) / 4;
+  const int64_t total = nwg * p.B * p.H;
+  if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)total), blk(256);
+  if (dtype == S3R_BF16)
+    hipLaunchKernelGGL((b16::select_b16_kernel<bf16_t>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total);
+  else
+    hipLaunchKernelGGL((b16::select_b16_kernel<f16_t>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total);
+  return check_launch("select_b16_kernel");
+}
+
+}  // namespace s3r

@@ -194,6 +194,35 @@ def test_select_matches_oracle(dtype, n, block, k):
     assert max_abs(lse, lse_ref) <= (1e-4 if dtype == torch.float32 else 2e-3)  # 16-bit: row sums are over rounded probabilities
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,k,with_invalid", [(96, 4, False), (1041, 32, False), (1041, 32, True), (200, 7, True), (16, 1, False),
+                                              (2000, 64, True), (70, 3, True)])
+def test_select_block16_matches_oracle(dtype, n, k, with_invalid):
+    """16-token blocks (the reference layer's own setting) run on the MFMA kernel that pairs query blocks: ragged
+    lengths, group tails (query-block counts that are not multiples of four), skipped and duplicated entries."""
+    h, block = 2, 16
+    nqb = -(-n // block)
+    q = _randn((1, h, n, 64), n, dtype, 0.5)
+    kk = _randn((1, h, n, 64), n + 1, dtype, 0.5)
+    v = _randn((1, h, n, 64), n + 2, dtype)
+    g = torch.Generator().manual_seed(n + k)
+    lo, hi = (-1, nqb + 1) if with_invalid else (0, nqb)
+    idx = torch.randint(lo, hi, (1, h, nqb, k), generator=g, dtype=torch.int32)
+    if with_invalid:
+        idx[0, 0, 0, :] = -1                    # a query block that attends nothing
+        if k > 1:
+            idx[0, 1, nqb - 1, 1] = idx[0, 1, nqb - 1, 0]   # a duplicate
+    o, lse = s3r.select_attn(q.to(DEV), kk.to(DEV), v.to(DEV), idx.to(DEV), block, return_lse=True)
+    o_ref, lse_ref = oracle.select_attention(q, kk, v, idx, block, out_dtype=torch.float32, return_lse=True)
+    assert o.dtype == dtype and o.shape == q.shape
+    assert max_abs(o, o_ref) <= TOL[dtype]
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert max_abs(lse.cpu()[fin], lse_ref[fin]) <= 2e-3
+    if with_invalid:
+        assert float(o[0, 0, :16].float().abs().max()) == 0.0
+
+
 def test_select_fixture(golden):
     q, k, v = (from_bf16_bits(golden[n]) for n in ("q", "k", "v"))
     idx = torch.from_numpy(golden["sel_idx"])
