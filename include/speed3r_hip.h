@@ -100,7 +100,7 @@ int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int
  *        entries < 0 or with idx*block >= N are skipped; duplicates are attended twice.
  *   o:   I/O dtype [B,H,N,D];  lse: optional fp32 [B,H,N] contiguous.
  * Keys beyond N in a partial last block are masked out; a query block with no valid entry
- * gives zeros.  block in {16,32,64}, D <= 64 (MFMA path: block == 64, D == 64, bf16/fp16).
+ * gives zeros.  block in {4,16,32,64}, D <= 64 (MFMA paths: block 64 or 16, D == 64, bf16/fp16, K <= 64).
  */
 int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx,
                     void* o, float* lse,
