@@ -50,6 +50,27 @@ def test_host_side_validation_returns_error_codes():
                              1, 1, 64, 64, 64, *([0] * 9), 7, None) == -2                           # unknown dtype
 
 
+def test_backward_entry_points_validate_on_the_host():
+    L = _lib.lib()
+    z3 = (0, 0, 0)
+    assert L.s3r_attn_bwd_delta(None, None, None, 1, 1, 64, 64, *z3, *z3, _lib.S3R_BF16, None) == _lib.S3R_ERR_BAD_ARG
+    one = ctypes.c_void_p(16)      # any non-null, 16-byte aligned address: validation never dereferences it
+    st = (64 * 64, 64 * 64, 64)
+
+    def bwd(dq=one, dk=one, dv=one, idx=None, lists=None, off=None, d=64, block=64, dtype=_lib.S3R_BF16, scale=0.125, q_st=st):
+        return L.s3r_attn_bwd(one, one, one, one, one, one, idx, lists, off, 0, dq, dk, dv, 1, 1, 64, 64, d, block, 4,
+                              *q_st, *st, *st, *st, *st, *st, *st, *z3, scale, dtype, None)
+
+    assert bwd(dq=None, dk=None, dv=None) == _lib.S3R_ERR_BAD_ARG           # no gradient requested
+    assert bwd(dk=None) == _lib.S3R_ERR_BAD_ARG                             # dk and dv come together
+    assert bwd(idx=one) == _lib.S3R_ERR_BAD_ARG                             # selection dk/dv without the key-centric lists
+    assert bwd(d=32) == _lib.S3R_ERR_UNSUPPORTED and bwd(block=16) == _lib.S3R_ERR_UNSUPPORTED
+    assert bwd(dtype=_lib.S3R_F32) == _lib.S3R_ERR_UNSUPPORTED and bwd(scale=0.0) == _lib.S3R_ERR_UNSUPPORTED
+    assert bwd(q_st=(64 * 64, 64 * 64, 1 << 20)) == _lib.S3R_ERR_UNSUPPORTED  # row stride beyond the 32-bit tile offsets
+    assert bwd(q_st=(64 * 64, 64 * 64, 60)) == _lib.S3R_ERR_BAD_ARG          # rows not 16-byte aligned
+    assert b"s3r_attn_bwd" in L.s3r_last_error()
+
+
 def test_operators_refuse_cpu_tensors():
     import speed3r_amd as s3r
 
