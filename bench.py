@@ -195,7 +195,7 @@ def main() -> int:
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path shards by head "
-              "without collectives, see DESIGN.md", file=sys.stderr)
+              "without collectives (heads are independent in every kernel)", file=sys.stderr)
         return 2
 
     import torch
