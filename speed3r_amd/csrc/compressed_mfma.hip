@@ -12,19 +12,19 @@
 // lane ^ 32, 32 of the tile's 64 keys in each lane's registers), base-2 online softmax in
 // fp32, P rounded to the I/O dtype, O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16.
 //
-// Fused selection.  Every lane keeps the exact top-K of the keys IT sees (half of each tile):
-// a descending sorted list of K keys, key = (sortable(bits(score)), Lk-1-col) in lexicographic order,
-// in registers.  Scores are first filtered against the score of the list's last entry (one
-// compare per score; survivors are appended to a small per-lane queue in LDS).  When some
-// lane's queue is more than half full, all lanes merge their queues into their lists with a
-// register-resident bitonic network (no divergence: every lane runs the same network on its
-// own data) and refresh their thresholds.  At the end the two lanes of a query merge their
-// lists and lane < 32 writes the K indices in descending key order.  The filter is
-// conservative (anything that could enter passes), the network compares full keys,
-// so the result is the same unique top-K as a sort of the whole row.
+// Selection without a score buffer (the top-k-only instance, KTOP > 0): two sweeps over the key tiles, K tiles by
+// direct transfers into an LDS ring.  Sweep 1 keeps, per lane, the K largest of its half-tile maxima; the K-th
+// largest of the two lanes' lists is a lower bound of the row's K-th largest score.  Sweep 2 recomputes the scores
+// and appends every score >= that threshold to a small per-lane queue in LDS (no branch).  Every lane keeps the
+// exact top-K of the keys IT sees (half of each tile): a descending sorted list of K keys,
+// key = (sortable(bits(score)), Lk-1-col) in lexicographic order, in registers.  When some lane's queue is nearly
+// full, all lanes merge their queues into their lists with a register-resident bitonic network (no divergence:
+// every lane runs the same network on its own data) and raise their thresholds to their lists' last entries.  At
+// the end the two lanes of a query merge their lists and lane < 32 writes the K indices in descending key order.
+// The filter is conservative (anything that could enter passes), the network compares full keys, so the result is
+// the same unique top-K as a sort of the whole row.
 #include "s3r_common.h"
 #include "attn_params.h"
-#include <type_traits>
 #include <type_traits>
 #include <utility>
 
@@ -258,13 +258,10 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
   };
 
   const int ntiles = (int)((Lk + 63) / 64);
-  // Fused selection, first pass: the maxima of the raw scores over groups of gsz key tiles (at most kGroups groups
-  // per row) go to the wave's queue memory, which is idle until the second pass: gmax[group * 32 + row], as 16-bit
-  // floats (the upper half of the fp32 pattern) rounded DOWN, so that a threshold taken from them is still a lower bound.
-  constexpr int kGroups = kQSlots * 8;  // 64 bytes per group in kQSlots * 512 bytes of queue
-  const int gsz = (ntiles + kGroups - 1) / kGroups;
-  uint16_t* gmax = FUSED ? reinterpret_cast<uint16_t*>(&queue[wave][0][0]) : nullptr;
-  float gm = -INFINITY;
+  // Fused selection, first sweep: per lane the K largest half-tile maxima, descending
+  float top[KL];
+#pragma unroll
+  for (int i = 0; i < KL; i++) top[i] = -INFINITY;
   if constexpr (!FUSED) {
   fetch(0);
   stash(0);
@@ -468,12 +465,13 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
               for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[kt][r]);
-            gm = fmaxf(gm, xh_max(mx));
-            if ((t + 1) % gsz == 0 || t + 1 == ntiles) {
-              const uint32_t u = __float_as_uint(gm);
-              const uint32_t down = (u >> 16) + (((u >> 31) != 0 && (u & 0xffffu) != 0) ? 1u : 0u);  // negative: one step further down
-              if (hh == 0) gmax[(t / gsz) * 32 + c] = (uint16_t)down;
-              gm = -INFINITY;
+            // this lane's maximum over its 32 keys of the tile goes into its descending list of the K largest such
+            // maxima (NaN never enters: fmaxf/fminf drop it)
+#pragma unroll
+            for (int i = 0; i < KL; i++) {
+              const float hi = fmaxf(top[i], mx);
+              mx = fminf(top[i], mx);
+              top[i] = hi;
             }
           } else {
             const uint32_t col0 = (uint32_t)start + 4 * hh;
@@ -511,26 +509,20 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
       }
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers issued past the last tile are done too
     };
-    // First sweep: the maximum raw score of every group of gsz key tiles, per query row.
+    // First sweep: every lane keeps the K largest of its half-tile maxima (maxima over 32 different keys each).
     sweep(std::false_type{});
-    // Threshold: the K-th largest group maximum of the row.  K different scores (one per group) are at least that
-    // large, so a score below it is not among the K largest, whatever the tie-break.  With fewer than K groups
-    // the threshold stays -inf and every score is a candidate.
+    // Threshold: the K-th largest of the row's half-tile maxima, i.e. of the union of the two lanes' lists.  K
+    // different scores (one per half tile) are at least that large, so a score below it is not among the K
+    // largest, whatever the tie-break.  With fewer than K half tiles it stays -inf and every score is a candidate.
+    // The K-th largest of two descending lists a, b is the largest min(a[i-1], b[K-i-1]) over the splits i.
     {
-      float top[KL];
+      float tau = fmaxf(top[KL - 1], __uint_as_float(xh_swap(__float_as_uint(top[KL - 1]))));  // splits i = K and i = 0
 #pragma unroll
-      for (int i = 0; i < KL; i++) top[i] = -INFINITY;
-      const int ngroups = (ntiles + gsz - 1) / gsz;
-      for (int g = 0; g < ngroups; g++) {
-        float x = __uint_as_float((uint32_t)gmax[g * 32 + c] << 16);
-#pragma unroll
-        for (int i = 0; i < KL; i++) {  // insertion into the descending list; NaN never enters (fmaxf/fminf drop it)
-          const float hi = fmaxf(top[i], x);
-          x = fminf(top[i], x);
-          top[i] = hi;
-        }
+      for (int i = 1; i < KL; i++) {
+        const float bi = __uint_as_float(xh_swap(__float_as_uint(top[KL - i - 1])));
+        tau = fmaxf(tau, fminf(top[i - 1], bi));
       }
-      thr0 = qvalid ? top[KL - 1] : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
+      thr0 = qvalid ? tau : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
       thr = thr0;
     }
     // Second sweep: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
