@@ -119,12 +119,12 @@ template <int N> __device__ __forceinline__ void merge_top_desc(key_t (&a)[N], c
 
 constexpr int kTile = 64 * 64;  // elements per LDS tile
 constexpr int kQCap = 16;       // width of the merge network that folds a lane's queue into its list
-// Top-k-only kernel, per list length: LDS queue slots per lane (the last one is the dump slot of non-survivors) and
-// K tiles in the LDS ring.  Up to 16: 28 KB of queues + 24 KB of tiles, three workgroups per compute unit;
-// above: 32 KB + 48 KB, two.
+// Top-k-only kernel: LDS queue slots per lane (the last one is the dump slot of non-survivors) and K tiles in the
+// LDS ring: 28 KB of queues + 24 KB of tiles, three workgroups per compute unit for every list length (the top-32
+// kernel reaches the 168 registers of that occupancy with 24 dwords spilled inside the queue drain, its rare path).
 template <int KTOP> struct TopkCfg {
-  static constexpr int kQSlots = KTOP <= 16 ? 14 : 16;
-  static constexpr int kRing = KTOP <= 16 ? 3 : 6;
+  static constexpr int kQSlots = 14;
+  static constexpr int kRing = 3;
 };
 template <> struct TopkCfg<0> {
   static constexpr int kQSlots = 1;
@@ -144,7 +144,7 @@ __device__ __forceinline__ void lds_reads_done(u32x4 (&a)[2][4]) {
 }
 
 template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */>
-__global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compressed_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(AttnParams p) {
   typedef typename Mma<E>::V8 V8;
   constexpr bool FUSED = KTOP > 0;
   constexpr int KL = FUSED ? KTOP : 1;  // list length per lane
@@ -245,11 +245,18 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
       merge_top_desc<kQCap>(wide, cand);
 #pragma unroll
       for (int i = 0; i < KL; i++) list[i] = wide[i];
-    } else {  // KL > kQCap: merge the candidates into the two (or more) halves' worth of list
-      key_t wide[KL];
+    } else {  // KL == 2 * kQCap, in place: the upper half U of the list beats its lower half M, and an element of
+      // M U cand outside that set's best kQCap cannot be among the KL best of the whole (kQCap of that set and, being
+      // below all of U, all kQCap of U are above it).  So: lower half <- best kQCap of M U cand, then one bitonic
+      // merge of the two sorted halves.
+      static_assert(KL == 2 * kQCap, "list lengths above the queue width are built for exactly twice that width");
+      key_t lower[kQCap];
 #pragma unroll
-      for (int i = 0; i < KL; i++) wide[i] = i < kQCap ? cand[i] : 0;
-      merge_top_desc<KL>(list, wide);
+      for (int i = 0; i < kQCap; i++) lower[i] = list[kQCap + i];
+      merge_top_desc<kQCap>(lower, cand);
+#pragma unroll
+      for (int i = 0; i < kQCap; i++) list[kQCap + i] = lower[kQCap - 1 - i];  // descending, then ascending: bitonic
+      bitonic_merge_desc<KL>(list);
     }
     qn = 0;
     // threshold = score of the list's last entry (key 0, a filler, maps to a NaN, which fmaxf drops: thr0 remains)
@@ -530,16 +537,26 @@ __global__ __launch_bounds__(256, (KTOP > 0 && KTOP <= 16) ? 3 : 2) void compres
     __syncthreads();  // every wave is done with the tile buffers of the first sweep
     sweep(std::true_type{});
     drain();
-    // the partner lane's list, then the K best of both, descending
-    key_t other[KL];
-#pragma unroll
-    for (int i = 0; i < KL; i++) {
-      const uint64_t bits = (uint64_t)__double_as_longlong(list[i]);
+    // the K best of this lane's list and the partner lane's, descending: max of entry i with the partner's entry
+    // K-1-i (a bitonic sequence), two entries at a time so that no second copy of the list is held, then one merge
+    auto partner = [&](key_t x) {
+      const uint64_t bits = (uint64_t)__double_as_longlong(x);
       const uint32_t lo = xh_swap((uint32_t)bits);
       const uint32_t hi = xh_swap((uint32_t)(bits >> 32));
-      other[i] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+      return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+    };
+    if constexpr (KL == 1) {
+      list[0] = __builtin_fmax(list[0], partner(list[0]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < KL / 2; i++) {
+        const key_t a = list[i], b = list[KL - 1 - i];
+        const key_t pa = partner(a), pb = partner(b);
+        list[i] = __builtin_fmax(a, pb);
+        list[KL - 1 - i] = __builtin_fmax(b, pa);
+      }
+      bitonic_merge_desc<KL>(list);
     }
-    merge_top_desc<KL>(list, other);
     if (qvalid && hh == 0) {
       int32_t* irow = p.topk_idx + (((int64_t)b * p.H + h) * Lq + qrow) * KL;
 #pragma unroll
