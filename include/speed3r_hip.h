@@ -169,7 +169,8 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
                     int dtype, void* stream);
 
 /*
- * Backward of the two attention operators (bf16/fp16, head_dim 64, block 64).
+ * Backward of the two attention operators (bf16/fp16, head_dim 64; selection blocks of 64 or 16 tokens, `block`
+ * is ignored when idx == NULL).
  * Replaces _topk_blocksparse_attention_bwd (pi3/models/sparse_attn/topk_blocksparse_attention.py:907-1038, kernels
  * backward_sum_o_do :132-170, backward_dkdv :558-712, backward_dq :722-850) and, with idx == NULL (every key tile),
  * _flash_attn_backward (pi3/models/sparse_attn/flash_attention_topk.py:204-630).
@@ -179,10 +180,10 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
  *   dv = P^T dout,  dS = scale * P * (dout v^T - delta),  dq = dS k,  dk = dS^T q;
  *   P and dS are rounded to the I/O dtype before the products, accumulation is fp32.
  *   lse: the forward's optional output (natural log, scaled scores), fp32 [B,H,Lq] contiguous.
- *   idx: the forward's block indices [B,H,ceil(Lq/64),K] (strides sib,sih,sim), or NULL for dense attention.
+ *   idx: the forward's block indices [B,H,ceil(Lq/block),K] (strides sib,sih,sim), or NULL for dense attention.
  *   kq_list, kq_off (needed for dk/dv when idx is given): for every (b,h) the query-block ids that list key block j,
  *     one entry per occurrence, ascending, are kq_list[(b*H+h)*list_stride + kq_off[(b*H+h)*(nkb+1) + j] ...
- *     kq_off[... + j+1]), nkb = ceil(Lk/64); entries of idx that are < 0 or >= nkb appear in no list
+ *     kq_off[... + j+1]), nkb = ceil(Lk/block); entries of idx that are < 0 or >= nkb appear in no list
  *     (reference count_query_fixedlen / reorder_topk_idx_fixedlen, :423-554).
  *   dq (layout strides sdq*), dk, dv (sdk*, sdv*): I/O dtype; dq == NULL or dk == dv == NULL skips that kernel.
  *   Every row of dq, dk, dv inside the tensors is written (zeros where nothing attends).

@@ -175,8 +175,8 @@ extern "C" int s3r_attn_bwd(const void* q, const void* k, const void* v, const v
   if ((dk == nullptr) != (dv == nullptr)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: dk and dv come together");
   if (idx != nullptr && dk != nullptr && (!kq_list || !kq_off)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: dk/dv of the selection branch need the key-centric lists");
   if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || (idx != nullptr && K <= 0)) return fail(S3R_ERR_BAD_ARG, "s3r_attn_bwd: non-positive size");
-  if ((dtype != S3R_BF16 && dtype != S3R_F16) || D != 64 || block != 64 || K > 64 || !(softmax_scale > 0.f))
-    return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd: built for bf16/fp16, head_dim 64, block 64, top-k <= 64, positive scale");
+  if ((dtype != S3R_BF16 && dtype != S3R_F16) || D != 64 || (idx != nullptr && block != 64 && block != 16) || K > 64 || !(softmax_scale > 0.f))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd: built for bf16/fp16, head_dim 64, block 64 or 16, top-k <= 64, positive scale");
   const int64_t lim = 1 << 20;
   if (sqm <= 0 || skn <= 0 || svn <= 0 || sgm <= 0 || sqm >= lim || skn >= lim || svn >= lim || sgm >= lim)
     return fail(S3R_ERR_UNSUPPORTED, "s3r_attn_bwd: row strides must be positive and below 2^20 elements");
@@ -186,7 +186,7 @@ extern "C" int s3r_attn_bwd(const void* q, const void* k, const void* v, const v
   BwdParams p = {};
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
   p.idx = idx; p.kq_list = kq_list; p.kq_off = kq_off; p.list_stride = list_stride;
-  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.K = K;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.K = K; p.block = idx != nullptr ? block : 64;
   p.sqb = sqb; p.sqh = sqh; p.sqm = sqm; p.skb = skb; p.skh = skh; p.skn = skn; p.svb = svb; p.svh = svh; p.svn = svn;
   p.sgb = sgb; p.sgh = sgh; p.sgm = sgm; p.sdqb = sdqb; p.sdqh = sdqh; p.sdqm = sdqm; p.sdkb = sdkb; p.sdkh = sdkh; p.sdkn = sdkn;
   p.sdvb = sdvb; p.sdvh = sdvh; p.sdvn = sdvn; p.sib = sib; p.sih = sih; p.sim = sim;

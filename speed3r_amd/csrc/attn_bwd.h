@@ -15,13 +15,14 @@ struct BwdParams {
   void* dq;                // nullptr: skip the dQ kernel
   void* dk;                // nullptr: skip the dK/dV kernel
   void* dv;
-  const int32_t* idx;      // [B,H,ceil(Lq/64),K] block indices of the forward, nullptr: every key tile (dense)
+  const int32_t* idx;      // [B,H,ceil(Lq/block),K] block indices of the forward, nullptr: every key tile (dense)
   const int32_t* kq_list;  // key-centric lists: query-block ids grouped by key block, [B,H,list_stride]
-  const int32_t* kq_off;   // [B,H,ceil(Lk/64)+1] offsets of each key block's list
+  const int32_t* kq_off;   // [B,H,ceil(Lk/block)+1] offsets of each key block's list
   int64_t list_stride;
   int B, H;
   int64_t Lq, Lk;
   int K;
+  int block;               // tokens per block of the selection branch: 64 or 16 (ignored without idx)
   int64_t sqb, sqh, sqm;
   int64_t skb, skh, skn;
   int64_t svb, svh, svn;

@@ -25,6 +25,13 @@
 //     dV^T += dO^T P and dK^T += Q^T dS read their A operands transposed from the same buffers.
 // Query rows beyond Lq have lse = +inf (P = 0), keys beyond Lk are masked (P = 0); rows past the end of a tensor are
 // never read (transfers re-read the last valid row).
+//
+// 16-token blocks (BLK = 16, the reference layer's own block size) run through the same kernels: a 32-row half tile
+// is then two 16-row blocks taken from two different lists (query blocks 2h, 2h+1 of the wave's 64 queries and entry t
+// of each one's index list in the dQ kernel; key blocks 2w, 2w+1 of the tile and entry t of each one's query-block
+// list in the dK/dV kernel).  A 32 x 32 product holds the two wanted 16 x 16 blocks on its diagonal; the other two
+// quadrants get P = 0.  Half h of the keys only meets half h of the queries, so the other half's products are not
+// issued at all.
 #include "select_common.h"
 #include "attn_bwd.h"
 
@@ -85,6 +92,25 @@ __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int f
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
                                                (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
     }
+  }
+}
+
+// The same for a half tile made of two 16-row blocks: instructions 0, 1 move block A, 2, 3 block B; rows are clamped
+// to last_a / last_b (relative to the block's first row).
+template <typename E, bool VSW>
+__device__ __forceinline__ void dma_rows16(const E* base_a, const E* base_b, uint32_t rowbytes, int last_a, int last_b, char* lds_half, int lane) {
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
+  const int lr = lane >> 3;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int ldsrow = 8 * i + lr;
+    const int last = i < 2 ? last_a : last_b;
+    int row = ldsrow & 15;
+    row = row < last ? row : last;
+    const int chunk = (lane & 7) ^ (VSW ? tsw(ldsrow) : (ldsrow & 7));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? ra : rb, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
+                                             (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
   }
 }
 
@@ -152,7 +178,7 @@ __device__ __forceinline__ void store_rows(const f32x16 (&acc)[2], E* rowptr, bo
 }
 
 // ---- dQ ----------------------------------------------------------------------------------------------------------
-template <typename E, bool DENSE>
+template <typename E, bool DENSE, int BLK>
 __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, int nqg, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[4 * kHalfBytes];
@@ -219,26 +245,47 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       for (int r = 0; r < 16; r++) dqt[qt][dt][r] = 0.f;
 
   // key tiles of this query block
+  static_assert(BLK == 64 || (BLK == 16 && !DENSE), "blocks of 64 tokens, or of 16 with an index list");
   int32_t my_idx = -1;
+  int32_t my16[4] = {-1, -1, -1, -1};  // BLK 16: entry `lane` of the lists of the wave's four query blocks
   uint64_t todo = 0;
   int ntiles;
   int dense_next = 0;
   if constexpr (DENSE) {
     ntiles = (int)((Lk + 63) >> 6);
-  } else {
+  } else if constexpr (BLK == 64) {
     const int32_t* idx_row = p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
     my_idx = lane < p.K ? idx_row[lane] : -1;
     todo = __ballot(my_idx >= 0 && (int64_t)my_idx * 64 < Lk);
     ntiles = __popcll(todo);
+  } else {
+    const int64_t nqb16 = (Lq + 15) >> 4;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int64_t qb16 = (int64_t)qb * 4 + s;
+      if (qb16 < nqb16 && lane < p.K) {
+        const int32_t v = (p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + qb16 * p.sim)[lane];
+        my16[s] = (v >= 0 && (int64_t)v * 16 < Lk) ? v : -1;
+      }
+    }
+    ntiles = p.K;  // entry t of all four lists makes tile t; entries that are skipped get P = 0
   }
-  auto pop = [&]() -> int64_t {  // start row of the next tile (callers pop exactly ntiles times)
+  auto pop = [&]() -> int64_t {  // start row of the next tile, BLK 16: its list position (callers pop exactly ntiles times)
     if constexpr (DENSE) {
       return (int64_t)(dense_next++) * 64;
-    } else {
+    } else if constexpr (BLK == 64) {
       const int t = __ffsll((unsigned long long)todo) - 1;
       todo &= todo - 1;
       return (int64_t)__builtin_amdgcn_readlane(my_idx, t) * 64;
+    } else {
+      return (int64_t)(dense_next++);
     }
+  };
+  // BLK 16: first key row and number of valid rows (0: skipped) of block `s` of tile t
+  auto sub_block = [&](int64_t t, int s, int64_t& start, int& nv) {
+    const int32_t v = __builtin_amdgcn_readlane(my16[s], (int)t);
+    start = v >= 0 ? (int64_t)v * 16 : 0;
+    nv = v >= 0 ? (int)(Lk - start < 16 ? Lk - start : 16) : 0;
   };
 
   const float scale = p.scale;
@@ -248,20 +295,41 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 
   auto fetch = [&](int64_t start, auto hf, int buf) {  // half HF of the tile at `start` -> buffers `buf`
     constexpr int HF = decltype(hf)::value;
-    const int last = (int)((Lk - start < 64 ? Lk - start : 64) - 1);
-    dma_rows<E, true>(kp + start * p.skn, krow, 32 * HF, last, k_buf[buf], lane, 0, 4);
-    dma_rows<E, false>(vp + start * p.svn, vrow, 32 * HF, last, v_buf[buf], lane, 0, 4);
+    if constexpr (BLK == 64) {
+      const int last = (int)((Lk - start < 64 ? Lk - start : 64) - 1);
+      dma_rows<E, true>(kp + start * p.skn, krow, 32 * HF, last, k_buf[buf], lane, 0, 4);
+      dma_rows<E, false>(vp + start * p.svn, vrow, 32 * HF, last, v_buf[buf], lane, 0, 4);
+    } else {
+      int64_t sa, sb;
+      int na, nb;
+      sub_block(start, 2 * HF, sa, na);
+      sub_block(start, 2 * HF + 1, sb, nb);
+      const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
+      dma_rows16<E, true>(kp + sa * p.skn, kp + sb * p.skn, krow, la, lb, k_buf[buf], lane);
+      dma_rows16<E, false>(vp + sa * p.svn, vp + sb * p.svn, vrow, la, lb, v_buf[buf], lane);
+    }
   };
   auto compute = [&](int64_t start, auto hf, int buf) {
     constexpr int HF = decltype(hf)::value;
-    const int nvalid = (int)(Lk - start < 64 ? Lk - start : 64);
+    int nvalid = 64;
+    int nv_mine = 16;  // BLK 16: valid keys of the block that this lane's query attends to in this half
+    if constexpr (BLK == 64) {
+      nvalid = (int)(Lk - start < 64 ? Lk - start : 64);
+    } else {
+      int64_t sa, sb;
+      int na, nb;
+      sub_block(start, 2 * HF, sa, na);
+      sub_block(start, 2 * HF + 1, sb, nb);
+      nv_mine = (c >> 4) ? nb : na;
+    }
     const bool ragged = nvalid < 64;
     V8 ak[4], av[4];
     read_rows<E, true>(k_buf[buf], c, hh, ak);
     read_rows<E, false>(v_buf[buf], c, hh, av);
     V8 ds[2][2];  // dS^T as B operand [qt][jj]
+    constexpr int QT0 = BLK == 64 ? 0 : HF, QT1 = BLK == 64 ? 2 : HF + 1;  // BLK 16: key half h meets query half h only
 #pragma unroll
-    for (int qt = 0; qt < 2; qt++) {
+    for (int qt = QT0; qt < QT1; qt++) {
       f32x16 st, dp;
 #pragma unroll
       for (int r = 0; r < 16; r++) { st[r] = 0.f; dp[r] = 0.f; }
@@ -271,10 +339,16 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(av[ks], bg[qt][ks], dp);
 #pragma unroll
       for (int r = 0; r < 16; r++) st[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));  // P^T
-      if (ragged) {  // keys beyond Lk carry no probability
+      if constexpr (BLK == 64) {
+        if (ragged) {  // keys beyond Lk carry no probability
+#pragma unroll
+          for (int r = 0; r < 16; r++)
+            if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) st[r] = 0.f;
+        }
+      } else {  // registers 0..7 are keys of block A, 8..15 of block B; this lane's query belongs to one of them
 #pragma unroll
         for (int r = 0; r < 16; r++)
-          if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) st[r] = 0.f;
+          if ((r >> 3) != (c >> 4) || 4 * hh + 8 * ((r >> 2) & 1) + (r & 3) >= nv_mine) st[r] = 0.f;
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[qt][r >> 3][r & 7] = (E)(st[r] * fmaf(dp[r], scale, -dlts[qt]));  // scale * P * (dP - delta)
@@ -286,7 +360,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 #pragma unroll
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-        for (int qt = 0; qt < 2; qt++) dqt[qt][dt] = Mma<E>::mma(kt[jj][dt], ds[qt][jj], dqt[qt][dt]);
+        for (int qt = QT0; qt < QT1; qt++) dqt[qt][dt] = Mma<E>::mma(kt[jj][dt], ds[qt][jj], dqt[qt][dt]);
   };
 
   if (ntiles > 0) {
@@ -320,7 +394,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 }
 
 // ---- dK, dV ------------------------------------------------------------------------------------------------------
-template <typename E, bool DENSE>
+template <typename E, bool DENSE, int BLK>
 __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, int nqb_all, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   constexpr int kTileBytes = 2 * kHalfBytes;  // a 64-row query tile
@@ -375,19 +449,34 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     for (int r = 0; r < 16; r++) { dkt[dt][r] = 0.f; dvt[dt][r] = 0.f; }
 
   // query blocks that attend to this key block
+  static_assert(BLK == 64 || (BLK == 16 && !DENSE), "blocks of 64 tokens, or of 16 with key-centric lists");
   int n_lists;
   const int32_t* list = nullptr;
+  const int32_t* list_b = nullptr;  // BLK 16: `list` belongs to this wave's first key block (2w of the tile), list_b to its second
+  int len_a = 0, len_b = 0;
   if constexpr (DENSE) {
     n_lists = nqb_all;
-  } else {
+  } else if constexpr (BLK == 64) {
     const int32_t* off = p.kq_off + ((int64_t)b * p.H + h) * (nkb + 1);
     const int32_t lo = off[kb], hi = off[kb + 1];
     n_lists = hi - lo;
     list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo;
+  } else {
+    const int64_t nkb16 = (Lk + 15) >> 4;
+    const int32_t* off = p.kq_off + ((int64_t)b * p.H + h) * (nkb16 + 1);
+    const int64_t ka = (int64_t)kb * 4 + 2 * wave;
+    const int32_t lo_a = ka < nkb16 ? off[ka] : 0, hi_a = ka < nkb16 ? off[ka + 1] : 0;
+    const int32_t lo_b = ka + 1 < nkb16 ? off[ka + 1] : 0, hi_b = ka + 1 < nkb16 ? off[ka + 2] : 0;
+    len_a = __builtin_amdgcn_readfirstlane(hi_a - lo_a);
+    len_b = __builtin_amdgcn_readfirstlane(hi_b - lo_b);
+    n_lists = len_a > len_b ? len_a : len_b;  // per wave: the two waves of a tile do not meet (see sync)
+    list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_a;
+    list_b = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_b;
   }
-  auto block_of = [&](int i) -> int64_t {
+  auto block_of = [&](int i) -> int64_t {  // BLK 16: the list position itself
     if constexpr (DENSE) return (int64_t)i;
-    else return (int64_t)__builtin_amdgcn_readfirstlane(list[i]);
+    else if constexpr (BLK == 64) return (int64_t)__builtin_amdgcn_readfirstlane(list[i]);
+    else return (int64_t)i;
   };
 
   const float scale = p.scale;
@@ -404,18 +493,39 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     char* qb = reinterpret_cast<char*>(BUF == 0 ? lds_q0 : lds_q1);
     char* gb = reinterpret_cast<char*>(BUF == 0 ? lds_g0 : lds_g1);
     float* sb = BUF == 0 ? lds_s0 : lds_s1;
-    const int64_t start = qblk * 64;
-    const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
+    if constexpr (BLK == 64) {
+      const int64_t start = qblk * 64;
+      const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
 #pragma unroll
-    for (int hf = 0; hf < 2; hf++) {
-      dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * hf, last, qb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
-      dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+      for (int hf = 0; hf < 2; hf++) {
+        dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * hf, last, qb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+        dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+      }
+      // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
+      // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
+      const int r = lane < last ? lane : last;
+      staged = ((wave == 0 ? lsep : dlp) + start)[r] * (wave == 0 ? kLog2e : scale);
+      staged_to = sb + 64 * wave + lane;
+    } else {
+      // this wave's half of the tile: 16 queries of entry `qblk` of each of its two lists (an exhausted list: any
+      // rows, lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
+      const int t = (int)qblk;
+      const int32_t ea = t < len_a ? __builtin_amdgcn_readfirstlane(list[t]) : -1;
+      const int32_t eb = t < len_b ? __builtin_amdgcn_readfirstlane(list_b[t]) : -1;
+      const int64_t sa = ea >= 0 ? (int64_t)ea * 16 : 0, sbk = eb >= 0 ? (int64_t)eb * 16 : 0;
+      const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
+      const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
+      const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
+      dma_rows16<E, true>(qp + sa * p.sqm, qp + sbk * p.sqm, qrow, la, lb, qb + wave * kHalfBytes, lane);
+      dma_rows16<E, true>(gp + sa * p.sgm, gp + sbk * p.sgm, grow, la, lb, gb + wave * kHalfBytes, lane);
+      const int j = lane & 31, j16 = j & 15;
+      const bool second = (j >> 4) != 0;
+      const int nmine = second ? nb : na;
+      const int64_t row = (second ? sbk : sa) + (j16 < nmine ? j16 : 0);
+      const float val = (hh == 0 ? lsep : dlp)[row] * (hh == 0 ? kLog2e : scale);
+      staged = (hh == 0 && j16 >= nmine) ? INFINITY : val;
+      staged_to = sb + 64 * hh + 32 * wave + j;
     }
-    // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
-    // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
-    const int r = lane < last ? lane : last;
-    staged = ((wave == 0 ? lsep : dlp) + start)[r] * (wave == 0 ? kLog2e : scale);
-    staged_to = sb + 64 * wave + lane;
   };
   auto publish = [&]() {
     if (staged_to != nullptr) *staged_to = staged;
@@ -424,9 +534,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   // One tile in three stages per 32-query half, issued so that the matrix products of one half run under the
   // vector work of the other: A = row reads + S, dP; B = P and dS from the per-query scalars; C = transposed reads +
   // dV^T, dK^T.
-  auto stage_a = [&](auto bufc, auto hf, f32x16& s, f32x16& dp) {
+  auto stage_a = [&](auto bufc, const int HF, f32x16& s, f32x16& dp) {
     constexpr int BUF = decltype(bufc)::value;
-    constexpr int HF = decltype(hf)::value;
     const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
     const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
     V8 aq[4], ag[4];
@@ -439,11 +548,10 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(ag[ks], bv[ks], dp);  // dP[q][key]
   };
-  auto stage_b = [&](int64_t qblk, auto bufc, auto hf, f32x16& s, f32x16& dp, V8 (&pb)[2], V8 (&db)[2]) {
+  auto stage_b = [&](int64_t qblk, auto bufc, const int HF, f32x16& s, f32x16& dp, V8 (&pb)[2], V8 (&db)[2]) {
     constexpr int BUF = decltype(bufc)::value;
-    constexpr int HF = decltype(hf)::value;
     const float* sb = (BUF == 0 ? lds_s0 : lds_s1) + 32 * HF;
-    const int nvalid = (int)(Lq - qblk * 64 < 64 ? Lq - qblk * 64 : 64);
+    const int nvalid = BLK == 64 ? (int)(Lq - qblk * 64 < 64 ? Lq - qblk * 64 : 64) : 64;  // BLK 16: lse = +inf does it
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(sb + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
@@ -460,15 +568,19 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       for (int r = 0; r < 16; r++)
         if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) s[r] = 0.f;
     }
+    if constexpr (BLK == 16) {  // registers 0..7 are queries of list A's block, 8..15 of list B's; this lane's key is in one
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        if ((r >> 3) != (c >> 4)) s[r] = 0.f;
+    }
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       pb[r >> 3][r & 7] = (E)s[r];
       db[r >> 3][r & 7] = (E)(s[r] * dp[r]);
     }
   };
-  auto stage_c = [&](auto bufc, auto hf, const V8 (&pb)[2], const V8 (&db)[2]) {
+  auto stage_c = [&](auto bufc, const int HF, const V8 (&pb)[2], const V8 (&db)[2]) {
     constexpr int BUF = decltype(bufc)::value;
-    constexpr int HF = decltype(hf)::value;
     const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
     const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
     V8 gt[2][2], qt[2][2];
@@ -483,22 +595,31 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       }
   };
   auto compute_tile = [&](int64_t qblk, auto bufc) {
-    f32x16 s0, dp0, s1, dp1;
-    V8 pb0[2], db0[2], pb1[2], db1[2];
-    stage_a(bufc, H0{}, s0, dp0);
-    stage_a(bufc, H1{}, s1, dp1);
-    stage_b(qblk, bufc, H0{}, s0, dp0, pb0, db0);
-    stage_c(bufc, H0{}, pb0, db0);
-    stage_b(qblk, bufc, H1{}, s1, dp1, pb1, db1);
-    stage_c(bufc, H1{}, pb1, db1);
+    if constexpr (BLK == 64) {
+      f32x16 s0, dp0, s1, dp1;
+      V8 pb0[2], db0[2], pb1[2], db1[2];
+      stage_a(bufc, 0, s0, dp0);
+      stage_a(bufc, 1, s1, dp1);
+      stage_b(qblk, bufc, 0, s0, dp0, pb0, db0);
+      stage_c(bufc, 0, pb0, db0);
+      stage_b(qblk, bufc, 1, s1, dp1, pb1, db1);
+      stage_c(bufc, 1, pb1, db1);
+    } else {  // this wave's keys only meet the queries of its own half of the tile
+      f32x16 s0, dp0;
+      V8 pb0[2], db0[2];
+      stage_a(bufc, wave, s0, dp0);
+      stage_b(qblk, bufc, wave, s0, dp0, pb0, db0);
+      stage_c(bufc, wave, pb0, db0);
+    }
   };
   // this wave's part of the tile has landed, its reads of the other buffer are done; after the barrier both hold
-  // for both waves
+  // for both waves (BLK 16: a wave only touches its own half of every buffer, so no barrier, and the two waves
+  // may walk lists of different lengths)
   auto sync = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     publish();
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
+    if constexpr (BLK == 64) __builtin_amdgcn_s_barrier();
   };
 
   if (n_lists > 0) {
@@ -535,16 +656,18 @@ int launch_attn_bwd(const BwdParams& p, int dtype, void* stream) {
   const int64_t total_q = nqg * p.B * p.H, total_k = nkb * p.B * p.H;
   if (total_q > 0x7fffffffLL || total_k > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "attention backward: grid too large");
   dim3 gq((unsigned)total_q), bq(256), gk((unsigned)total_k), bk(128);
-#define S3R_BWD_LAUNCH(E)                                                                                                   \
-  do {                                                                                                                      \
-    if (p.dq != nullptr) {                                                                                                  \
-      if (dense) hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, true>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);     \
-      else hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, false>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);          \
-    }                                                                                                                       \
-    if (p.dk != nullptr) {                                                                                                  \
-      if (dense) hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, true>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);   \
-      else hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, false>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);        \
-    }                                                                                                                       \
+#define S3R_BWD_LAUNCH(E)                                                                                                       \
+  do {                                                                                                                          \
+    if (p.dq != nullptr) {                                                                                                      \
+      if (dense) hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, true, 64>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);     \
+      else if (p.block == 16) hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, false, 16>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q); \
+      else hipLaunchKernelGGL((bwd::bwd_dq_kernel<E, false, 64>), gq, bq, 0, st, p, (int)nqb, (int)nqg, (int)total_q);          \
+    }                                                                                                                           \
+    if (p.dk != nullptr) {                                                                                                      \
+      if (dense) hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, true, 64>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);   \
+      else if (p.block == 16) hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, false, 16>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k); \
+      else hipLaunchKernelGGL((bwd::bwd_dkdv_kernel<E, false, 64>), gk, bk, 0, st, p, (int)nkb, (int)nqb, (int)total_k);        \
+    }                                                                                                                           \
   } while (0)
   if (dtype == S3R_BF16) S3R_BWD_LAUNCH(bf16_t);
   else S3R_BWD_LAUNCH(f16_t);

@@ -10,7 +10,7 @@ Differences, all on the host side of the operator boundary:
   (or in its own kernel where that is not built), writing ``[B, N, C]`` for ``proj``;
 * when a gradient is wanted (grad mode on and the input or a parameter requires grad) the layer runs as a
   differentiable composition instead: the two attention operators with their backward kernels (bf16/fp16,
-  head_dim 64, block 64), pooling, norm/RoPE and merge as torch expressions;
+  head_dim 64, blocks of 64 or 16 tokens), pooling, norm/RoPE and merge as torch expressions;
 * ``N`` need not be a multiple of the block: the last block pools its valid tokens, its keys beyond ``N`` are
   masked and its query rows beyond ``N`` do not exist (the reference raises for such ``N``);
 * the top-k count, 32 in the reference, is a constructor argument.

@@ -283,8 +283,8 @@ def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: to
 # ---- backward of the two attention operators --------------------------------------------------------------------
 
 def bwd_supported(q: torch.Tensor, block: int = 64) -> bool:
-    """The backward kernels are built for bf16/fp16, head_dim 64, block 64."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] == 64 and block == 64
+    """The backward kernels are built for bf16/fp16, head_dim 64, blocks of 64 or 16 tokens."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] == 64 and block in (64, 16)
 
 
 def key_block_lists(idx: torch.Tensor, n_key_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -326,7 +326,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
     selection attention over the blocks of ``idx`` ([B,H,Nq_blocks,K] int32), or dense attention (``idx=None``).
     ``delta`` (:func:`attn_bwd_delta`) and ``key_lists`` (:func:`key_block_lists`) are computed here unless given."""
     _need_device(q, k, v, o, dout, lse)
-    assert bwd_supported(q, block), "attention backward: built for bf16/fp16, head_dim 64, block 64"
+    assert bwd_supported(q, block), "attention backward: built for bf16/fp16, head_dim 64, block 64 or 16"
     q, k, v, o, dout = (_last_contig(t) for t in (q, k, v, o, dout))
     lse = lse.contiguous()
     b, h, lq, d = q.shape
@@ -337,12 +337,12 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
     dq = torch.empty_like(q, memory_format=torch.contiguous_format) if need_dq else None
     dk = torch.empty_like(k, memory_format=torch.contiguous_format) if need_dkv else None
     dv = torch.empty_like(v, memory_format=torch.contiguous_format) if need_dkv else None
-    nkb = -(-lk // 64)
+    nkb = -(-lk // block)
     lists = offs = None
     kk = 0
     if idx is not None:
         idx = _last_contig(idx)
-        assert idx.dtype == torch.int32 and idx.shape[:3] == (b, h, -(-lq // 64))
+        assert idx.dtype == torch.int32 and idx.shape[:3] == (b, h, -(-lq // block))
         kk = idx.shape[3]
         if need_dkv:
             lists, offs = key_lists if key_lists is not None else key_block_lists(idx, nkb)
@@ -415,7 +415,7 @@ def select_attn_autograd(q, k, v, idx, block, softmax_scale=None):
     if not _wants_grad(q, k, v):
         return select_attn(q, k, v, idx, block, softmax_scale)
     if not bwd_supported(q, block):
-        raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64, block 64 only")
+        raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64, blocks of 64 or 16 tokens")
     return _SelectAttnFn.apply(q, k, v, idx, block, softmax_scale)
 
 

@@ -64,7 +64,8 @@ def test_backward_entry_points_validate_on_the_host():
     assert bwd(dq=None, dk=None, dv=None) == _lib.S3R_ERR_BAD_ARG           # no gradient requested
     assert bwd(dk=None) == _lib.S3R_ERR_BAD_ARG                             # dk and dv come together
     assert bwd(idx=one) == _lib.S3R_ERR_BAD_ARG                             # selection dk/dv without the key-centric lists
-    assert bwd(d=32) == _lib.S3R_ERR_UNSUPPORTED and bwd(block=16) == _lib.S3R_ERR_UNSUPPORTED
+    assert bwd(d=32) == _lib.S3R_ERR_UNSUPPORTED
+    assert bwd(idx=one, lists=one, off=one, block=32) == _lib.S3R_ERR_UNSUPPORTED   # selection blocks of 64 or 16 tokens
     assert bwd(dtype=_lib.S3R_F32) == _lib.S3R_ERR_UNSUPPORTED and bwd(scale=0.0) == _lib.S3R_ERR_UNSUPPORTED
     assert bwd(q_st=(64 * 64, 64 * 64, 1 << 20)) == _lib.S3R_ERR_UNSUPPORTED  # row stride beyond the 32-bit tile offsets
     assert bwd(q_st=(64 * 64, 64 * 64, 60)) == _lib.S3R_ERR_BAD_ARG          # rows not 16-byte aligned

@@ -84,6 +84,41 @@ def test_selection_backward_with_skips_duplicates_and_unattended_keys():
     assert float(dk[0, :, 512:].abs().max()) == 0.0 and float(dv[0, :, 512:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,kk", [(256, 4), (1000, 8), (1041, 32), (64, 2), (40, 1), (2100, 16)])
+def test_selection_backward_with_16_token_blocks_matches_oracle(dtype, n, kk):
+    """Block 16, the reference layer's own setting (sparse_attention.py:73,98): sequence lengths that are no multiple
+    of 16 or of 64, so ragged blocks and partly filled 64-row tiles are covered."""
+    b, h = 1, 2
+    nqb = -(-n // 16)
+    q, k, v, g = (_randn((b, h, n, 64), 130 + i, dtype, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb, 140 + n)
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 16, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd, 16)
+    wq, wk, wv = oracle.select_attention_grads_autograd(q, k, v, idx, 16, g)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+
+
+def test_selection_backward_with_16_token_blocks_skips_duplicates_and_popular_keys():
+    b, h, n, kk = 1, 2, 400, 4
+    nqb = n // 16
+    q, k, v, g = (_randn((b, h, n, 64), 150 + i, torch.bfloat16, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb - 3, 155, lo=-1)       # -1 entries; the last three key blocks are never attended
+    idx[0, 0, 2] = torch.tensor([3, 3, 3, 1])                   # duplicates
+    idx[0, 1, 4] = -1                                           # a query block that attends nothing
+    idx[0, 1, 5, 0] = nqb + 3                                   # beyond the sequence: skipped
+    idx[0, 0, :, 1] = 7                                         # one key block on every list: lists of unequal length
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 16, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd, 16)
+    mult = oracle.block_multiplicity(idx, n, 16)
+    wq, wk, wv, _, _ = oracle.attention_grads_formula(q, k, v, g, mult)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+    assert float(dq[0, 1, 64:80].abs().max()) == 0.0                      # the empty query block
+    assert float(dk[0, :, 16 * (nqb - 3):].abs().max()) == 0.0 and float(dv[0, :, 16 * (nqb - 3):].abs().max()) == 0.0
+
+
 def test_operators_are_differentiable_like_the_reference_ones():
     b, h, n = 1, 2, 512
     q, k, v = (_randn((b, h, n, 64), 60 + i, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for i in range(3))

@@ -66,7 +66,7 @@ def test_layer_without_norm_and_positions():
 
 
 def test_layer_refuses_gradients_where_no_backward_kernel_is_built():
-    m = _make(128, 2, 4, 2, torch.bfloat16, seed=7).to(DEV)      # block 16: the backward kernels are built for block 64
+    m = _make(128, 2, 2, 2, torch.bfloat16, seed=7).to(DEV)      # block 4: the backward kernels are built for blocks 64 and 16
     x = torch.randn((1, 128, 128), device=DEV, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError):
         m(x)                      # parameters require grad and grad mode is on
@@ -108,9 +108,9 @@ def test_norm_rope_kernel_matches_the_torch_modules(dtype, with_norm, with_pos):
         assert (got == want).float().mean().item() >= 0.97
 
 
-@pytest.mark.parametrize("n", [320, 200])
-def test_layer_gradients_match_autograd_through_the_oracle(n):
-    b, dim, heads, block_size, topk = 1, 128, 2, 8, 2
+@pytest.mark.parametrize("n,block_size,topk", [(320, 8, 2), (200, 8, 2), (320, 4, 4), (200, 4, 4)])
+def test_layer_gradients_match_autograd_through_the_oracle(n, block_size, topk):
+    b, dim, heads = 1, 128, 2
     m = _make(dim, heads, block_size, topk, torch.bfloat16, seed=40 + n)
     g = torch.Generator().manual_seed(41 + n)
     x = torch.randn((b, n, dim), generator=g).to(torch.bfloat16)
