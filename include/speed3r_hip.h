@@ -188,6 +188,18 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
  *   dq (layout strides sdq*), dk, dv (sdk*, sdv*): I/O dtype; dq == NULL or dk == dv == NULL skips that kernel.
  *   Every row of dq, dk, dv inside the tensors is written (zeros where nothing attends).
  */
+/*
+ * Key-centric lists for s3r_attn_bwd from the forward's index tensor.
+ * Replaces count_query_fixedlen, the stable argsort and reorder_topk_idx_fixedlen of the reference's backward
+ * (pi3/models/sparse_attn/topk_blocksparse_attention.py:423-554).
+ *   idx: [B,H,nqb,K] int32 (strides sib,sih,sim, last dimension contiguous); nkb: number of key blocks.
+ *   kq_off: [B,H,nkb+1] int32, contiguous; kq_list: [B,H,list_stride] int32, list_stride >= nqb*K.
+ * Block j's list of (b,h) = kq_list[(b*H+h)*list_stride + kq_off[..j] ... kq_off[..j+1]): the query-block ids whose
+ * index row names j, one entry per occurrence, ascending.  Entries of idx < 0 or >= nkb appear in no list; the part
+ * of kq_list behind kq_off[..nkb] is left as it was.  No workspace; the result does not depend on the run.
+ */
+int s3r_key_block_lists(const int32_t* idx, int32_t* kq_list, int32_t* kq_off, int B, int H, int64_t nqb, int K, int64_t nkb,
+                        int64_t sib, int64_t sih, int64_t sim, int64_t list_stride, void* stream);
 int s3r_attn_bwd_delta(const void* o, const void* dout, float* delta, int B, int H, int64_t N, int D,
                        int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
                        int dtype, void* stream);

@@ -38,6 +38,7 @@ SIGNATURES = {
                                 *_i64x3, *_i64x3, *_i64x3, c_int, c_void_p]),
     "s3r_attn_bwd_delta": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, *_i64x3, *_i64x3,
                                    c_int, c_void_p]),
+    "s3r_key_block_lists": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int64, *_i64x3, c_int64, c_void_p]),
     "s3r_attn_bwd": (c_int, [c_void_p] * 6 + [c_void_p, c_void_p, c_void_p, c_int64] + [c_void_p] * 3
                      + [c_int, c_int, c_int64, c_int64, c_int, c_int, c_int]
                      + _i64x3 * 8 + [c_float, c_int, c_void_p]),

@@ -161,6 +161,15 @@ extern "C" int s3r_attn_bwd_delta(const void* o, const void* dout, float* delta,
   return launch_bwd_delta(o, dout, delta, B, H, N, sob, soh, son, sdb, sdh, sdn, dtype, stream);
 }
 
+extern "C" int s3r_key_block_lists(const int32_t* idx, int32_t* kq_list, int32_t* kq_off, int B, int H, int64_t nqb, int K, int64_t nkb,
+                                   int64_t sib, int64_t sih, int64_t sim, int64_t list_stride, void* stream) {
+  if (!idx || !kq_list || !kq_off) return fail(S3R_ERR_BAD_ARG, "s3r_key_block_lists: null pointer");
+  if (B <= 0 || H <= 0 || nqb <= 0 || K <= 0 || nkb <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_key_block_lists: non-positive size");
+  if (nqb * K > 0x7fffffffLL || nkb >= 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_key_block_lists: more than 2^31 entries per head");
+  if (list_stride < nqb * K) return fail(S3R_ERR_BAD_ARG, "s3r_key_block_lists: list_stride below nqb * K");
+  return launch_key_block_lists(idx, kq_list, kq_off, B, H, nqb, K, nkb, sib, sih, sim, list_stride, stream);
+}
+
 extern "C" int s3r_attn_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse, const float* delta,
                             const int32_t* idx, const int32_t* kq_list, const int32_t* kq_off, int64_t list_stride,
                             void* dq, void* dk, void* dv,

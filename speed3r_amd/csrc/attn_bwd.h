@@ -35,6 +35,8 @@ struct BwdParams {
 };
 
 int launch_attn_bwd(const BwdParams& p, int dtype, void* stream);
+int launch_key_block_lists(const int32_t* idx, int32_t* kq_list, int32_t* kq_off, int B, int H, int64_t nqb, int K, int64_t nkb,
+                           int64_t sib, int64_t sih, int64_t sim, int64_t list_stride, void* stream);
 int launch_bwd_delta(const void* o, const void* dout, float* delta, int B, int H, int64_t N, int64_t sob, int64_t soh, int64_t son,
                      int64_t sdb, int64_t sdh, int64_t sdn, int dtype, void* stream);
 

@@ -289,19 +289,21 @@ def bwd_supported(q: torch.Tensor, block: int = 64) -> bool:
 
 def key_block_lists(idx: torch.Tensor, n_key_blocks: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Key-centric view of the index tensor ``[B,H,Nq_blocks,K]``: for every (b, h) the query-block ids grouped by
-    the key block they list, one entry per occurrence, ascending within a group (stable), and the group offsets
-    ``[B,H,n_key_blocks+1]``; entries < 0 or >= n_key_blocks appear in no group.  Same construction as the
-    reference's count + stable argsort (topk_blocksparse_attention.py:423-554), with torch device routines."""
+    the key block they list, one entry per occurrence, ascending within a group, ``[B,H,Nq_blocks*K]`` int32, and the
+    group offsets ``[B,H,n_key_blocks+1]``; entries < 0 or >= n_key_blocks appear in no group (the tail of the list
+    tensor behind the last offset is then unspecified).  The reference's count + stable argsort + reorder
+    (topk_blocksparse_attention.py:423-554)."""
+    _need_device(idx)
+    assert idx.dtype == torch.int32 and idx.dim() == 4 and n_key_blocks > 0
+    idx = _last_contig(idx)
     b, h, nqb, kk = idx.shape
-    flat = idx.reshape(b, h, nqb * kk).long()
-    keys = torch.where((flat >= 0) & (flat < n_key_blocks), flat, torch.full_like(flat, n_key_blocks))
-    order = torch.argsort(keys, dim=-1, stable=True)
-    qblk = torch.div(order, kk, rounding_mode="floor").to(torch.int32).contiguous()
-    counts = torch.zeros((b, h, n_key_blocks + 1), dtype=torch.int64, device=idx.device)
-    counts.scatter_add_(-1, keys, torch.ones_like(keys))
-    off = torch.zeros((b, h, n_key_blocks + 1), dtype=torch.int32, device=idx.device)
-    off[..., 1:] = counts[..., :n_key_blocks].cumsum(-1).to(torch.int32)
-    return qblk, off
+    lists = torch.empty((b, h, nqb * kk), dtype=torch.int32, device=idx.device)
+    off = torch.empty((b, h, n_key_blocks + 1), dtype=torch.int32, device=idx.device)
+    with torch.cuda.device(idx.device):
+        rc = _lib.lib().s3r_key_block_lists(idx.data_ptr(), lists.data_ptr(), off.data_ptr(), b, h, nqb, kk, n_key_blocks,
+                                            idx.stride(0), idx.stride(1), idx.stride(2), nqb * kk, _stream(idx))
+    _lib.check(rc, "s3r_key_block_lists")
+    return lists, off
 
 
 def attn_bwd_delta(o: torch.Tensor, dout: torch.Tensor) -> torch.Tensor:

@@ -119,6 +119,35 @@ def test_selection_backward_with_16_token_blocks_skips_duplicates_and_popular_ke
     assert float(dk[0, :, 16 * (nqb - 3):].abs().max()) == 0.0 and float(dv[0, :, 16 * (nqb - 3):].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("b,h,nqb,kk,nkb,hot", [(2, 3, 37, 4, 37, 0), (1, 2, 300, 8, 300, 1), (1, 1, 2600, 4, 650, 2),
+                                                (1, 2, 9000, 2, 40, 3), (1, 1, 1, 1, 1, 0), (1, 2, 70, 64, 70, 0)])
+def test_key_block_lists_match_plain_loops(b, h, nqb, kk, nkb, hot):
+    """The device lists against the oracle's plain loops: entries outside [0, nkb), duplicates, lists of up to 512
+    entries (sorted by one wavefront), of more (by a workgroup in LDS; hot == 2) and of more than 8192 (in global
+    memory; hot == 3), and the same bits on a second run (the atomic order of the fill must not show)."""
+    gen = torch.Generator().manual_seed(22 + nqb)
+    idx = torch.randint(-2, nkb + 2, (b, h, nqb, kk), generator=gen, dtype=torch.int32)
+    if hot >= 1:
+        idx[0, 0, :, 0] = 5                      # a key block on every index row
+    if hot >= 2:
+        idx[0, 0, ::3, 1] = 5                    # ... twice on every third
+    if hot >= 3:
+        idx[0, 1] = 7                            # nqb * K = 18 000 entries in one list
+    idx[-1, -1, nqb // 2] = 1
+    lists, off = ops.key_block_lists(idx.to(DEV), nkb)
+    lists2, off2 = ops.key_block_lists(idx.to(DEV), nkb)
+    want = oracle.key_block_lists(idx, nkb)
+    assert lists.dtype == torch.int32 and off.dtype == torch.int32 and off.shape == (b, h, nkb + 1)
+    assert torch.equal(off, off2)
+    off, lists, lists2 = off.cpu(), lists.cpu(), lists2.cpu()
+    for bh in range(b * h):
+        o = off.view(b * h, nkb + 1)[bh].tolist()
+        flat = lists.view(b * h, -1)[bh].tolist()
+        assert o[0] == 0 and flat[:o[-1]] == lists2.view(b * h, -1)[bh].tolist()[:o[-1]]
+        for j in range(nkb):
+            assert flat[o[j]:o[j + 1]] == want[bh][j], (bh, j)
+
+
 def test_operators_are_differentiable_like_the_reference_ones():
     b, h, n = 1, 2, 512
     q, k, v = (_randn((b, h, n, 64), 60 + i, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for i in range(3))

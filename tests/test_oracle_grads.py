@@ -83,19 +83,17 @@ def test_gradient_invariants():
     assert max_abs(dq, dq2) <= 1e-10 and max_abs(dk, dk2) <= 1e-10
 
 
-def test_key_block_lists_of_the_host_code_match_plain_loops():
-    from speed3r_amd.sparse_attn.ops import key_block_lists
-
+def test_key_block_lists_of_the_oracle_hold_every_valid_entry_once_and_in_order():
     gen = torch.Generator().manual_seed(22)
     b, h, nqb, kk, nkb = 2, 3, 37, 4, 37
     idx = torch.randint(-2, nkb + 2, (b, h, nqb, kk), generator=gen, dtype=torch.int32)
     idx[1, 2, 5] = torch.tensor([7, 7, 7, 1])
-    lists, off = key_block_lists(idx, nkb)
-    want = oracle.key_block_lists(idx, nkb)
-    assert lists.dtype == torch.int32 and off.dtype == torch.int32 and off.shape == (b, h, nkb + 1)
+    got = oracle.key_block_lists(idx, nkb)
+    assert got[1 * h + 2][7].count(5) == 3 and got[1 * h + 2][1].count(5) == 1
     for bh in range(b * h):
-        o = off.view(b * h, nkb + 1)[bh].tolist()
-        flat = lists.view(b * h, -1)[bh].tolist()
-        assert o[0] == 0
+        rows = idx.view(b * h, nqb, kk)[bh]
+        assert sum(len(l) for l in got[bh]) == int(((rows >= 0) & (rows < nkb)).sum())
         for j in range(nkb):
-            assert flat[o[j]:o[j + 1]] == want[bh][j], (bh, j)
+            assert got[bh][j] == sorted(got[bh][j])
+            for m in set(got[bh][j]):
+                assert got[bh][j].count(m) == int((rows[m] == j).sum())
