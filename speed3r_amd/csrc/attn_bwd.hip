@@ -410,7 +410,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const int hh = lane >> 5;
   const int c = lane & 31;
 
-  const int w = blockIdx.x;
+  // With lists the grid has two passes over the key blocks: the first (workgroups [0, total_wg)) takes the blocks whose
+  // lists are long, the second the others, so the longest lists of a skewed index tensor start first instead of
+  // wherever their key block falls in the launch order.
+  const bool long_pass = DENSE || (int)blockIdx.x < total_wg;
+  const int w = (int)blockIdx.x < total_wg ? (int)blockIdx.x : (int)blockIdx.x - total_wg;
   const int xcd = w & 7, slot = w >> 3;
   const int per = total_wg >> 3, rem = total_wg & 7;
   const int vid = xcd * per + (xcd < rem ? xcd : rem) + slot;
@@ -420,6 +424,20 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const int h = bh - b * p.H;
 
   const int64_t Lq = p.Lq, Lk = p.Lk;
+  if constexpr (!DENSE) {
+    const int64_t nkbl = (Lk + BLK - 1) / BLK;
+    const int32_t* off = p.kq_off + ((int64_t)b * p.H + h) * (nkbl + 1);
+    int len;
+    if constexpr (BLK == 64) {
+      len = off[kb + 1] - off[kb];
+    } else {  // the longer of this wave's two lists (the waves of a workgroup are independent)
+      const int64_t ka = (int64_t)kb * 4 + 2 * wave;
+      const int la = ka < nkbl ? off[ka + 1] - off[ka] : 0, lb = ka + 1 < nkbl ? off[ka + 2] - off[ka + 1] : 0;
+      len = la > lb ? la : lb;
+    }
+    len = __builtin_amdgcn_readfirstlane(len);
+    if ((len > 4 * p.K) != long_pass) return;
+  }
   const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
   const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
   const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
@@ -473,9 +491,20 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_a;
     list_b = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_b;
   }
+  // List entries come 64 at a time (lane l holds entry base + l), so the latency of the list read is paid once per
+  // 64 tiles and not in front of every tile's transfers.  The lists are walked front to back.
+  int32_t held_a = -1, held_b = -1;
+  int base_a = -64, base_b = -64;
+  auto entry = [&](const int32_t* lst, int len, int32_t& held, int& base, int i) -> int32_t {
+    if (i >= base + 64) {
+      base = i & ~63;
+      held = base + lane < len ? lst[base + lane] : -1;
+    }
+    return __builtin_amdgcn_readlane(held, i - base);
+  };
   auto block_of = [&](int i) -> int64_t {  // BLK 16: the list position itself
     if constexpr (DENSE) return (int64_t)i;
-    else if constexpr (BLK == 64) return (int64_t)__builtin_amdgcn_readfirstlane(list[i]);
+    else if constexpr (BLK == 64) return (int64_t)entry(list, n_lists, held_a, base_a, i);
     else return (int64_t)i;
   };
 
@@ -510,8 +539,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       // this wave's half of the tile: 16 queries of entry `qblk` of each of its two lists (an exhausted list: any
       // rows, lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
       const int t = (int)qblk;
-      const int32_t ea = t < len_a ? __builtin_amdgcn_readfirstlane(list[t]) : -1;
-      const int32_t eb = t < len_b ? __builtin_amdgcn_readfirstlane(list_b[t]) : -1;
+      const int32_t ea = t < len_a ? entry(list, len_a, held_a, base_a, t) : -1;
+      const int32_t eb = t < len_b ? entry(list_b, len_b, held_b, base_b, t) : -1;
       const int64_t sa = ea >= 0 ? (int64_t)ea * 16 : 0, sbk = eb >= 0 ? (int64_t)eb * 16 : 0;
       const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
       const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
@@ -655,7 +684,8 @@ int launch_attn_bwd(const BwdParams& p, int dtype, void* stream) {
   const int64_t nqg = (nqb + 3) / 4;
   const int64_t total_q = nqg * p.B * p.H, total_k = nkb * p.B * p.H;
   if (total_q > 0x7fffffffLL || total_k > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "attention backward: grid too large");
-  dim3 gq((unsigned)total_q), bq(256), gk((unsigned)total_k), bk(128);
+  if (!dense && 2 * total_k > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "attention backward: grid too large");
+  dim3 gq((unsigned)total_q), bq(256), gk((unsigned)(dense ? total_k : 2 * total_k)), bk(128);
 #define S3R_BWD_LAUNCH(E)                                                                                                       \
   do {                                                                                                                          \
     if (p.dq != nullptr) {                                                                                                      \
