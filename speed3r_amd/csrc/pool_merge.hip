@@ -9,7 +9,7 @@
 
 namespace s3r {
 
-template <typename T>
+template <typename T, int U>
 __global__ __launch_bounds__(256) void pool_mean_kernel(
     const T* __restrict__ x, T* __restrict__ y, int H, int64_t N, int D, int block, int64_t Nc,
     int64_t total, int64_t sxb, int64_t sxh, int64_t sxn, int64_t syb, int64_t syh, int64_t syn) {
@@ -32,17 +32,18 @@ __global__ __launch_bounds__(256) void pool_mean_kernel(
   float acc[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; i++) acc[i] = 0.f;
-  // batches of 8 loads issued back to back (rows beyond the block re-read its last row and are not added),
-  // so that 8 KB per wave are in flight instead of one load at a time
-  for (int r = r0; r < nvalid; r += 8 * rpw) {
-    uint4 raw[8];
+  // batches of U loads issued back to back (rows beyond the block re-read its last row and are not added),
+  // so that up to 8 KB per wave are in flight instead of one load at a time; U = 8 or, for blocks below 8 wave-wide
+  // loads, the number that covers the block
+  for (int r = r0; r < nvalid; r += U * rpw) {
+    uint4 raw[U];
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
+    for (int u = 0; u < U; u++) {
       const int rr = r + u * rpw;
       raw[u] = *reinterpret_cast<const uint4*>(base + (int64_t)(rr < nvalid ? rr : nvalid - 1) * sxn);
     }
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
+    for (int u = 0; u < U; u++) {
       const T* e = reinterpret_cast<const T*>(&raw[u]);
       const bool keep = r + u * rpw < nvalid;
 #pragma unroll
@@ -122,12 +123,20 @@ extern "C" int s3r_pool_mean(const void* x, void* y, int B, int H, int64_t N, in
   if (nwg > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_pool_mean: too many blocks");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)nwg), blk(256);
-  if (dtype == S3R_F32)
-    hipLaunchKernelGGL(pool_mean_kernel<float>, grid, blk, 0, st, (const float*)x, (float*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
-  else if (dtype == S3R_BF16)
-    hipLaunchKernelGGL(pool_mean_kernel<bf16_t>, grid, blk, 0, st, (const bf16_t*)x, (bf16_t*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
-  else
-    hipLaunchKernelGGL(pool_mean_kernel<f16_t>, grid, blk, 0, st, (const f16_t*)x, (f16_t*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn);
+  const int loads = (block * lpr + 63) / 64;  // wave-wide loads that cover one block
+#define S3R_POOL(T, U) hipLaunchKernelGGL((pool_mean_kernel<T, U>), grid, blk, 0, st, (const T*)x, (T*)y, H, N, D, block, Nc, total, sxb, sxh, sxn, syb, syh, syn)
+#define S3R_POOL_T(T)                    \
+  do {                                   \
+    if (loads <= 1) S3R_POOL(T, 1);      \
+    else if (loads <= 2) S3R_POOL(T, 2); \
+    else if (loads <= 4) S3R_POOL(T, 4); \
+    else S3R_POOL(T, 8);                 \
+  } while (0)
+  if (dtype == S3R_F32) S3R_POOL_T(float);
+  else if (dtype == S3R_BF16) S3R_POOL_T(bf16_t);
+  else S3R_POOL_T(f16_t);
+#undef S3R_POOL_T
+#undef S3R_POOL
   return check_launch("s3r_pool_mean");
 }
 

@@ -30,7 +30,8 @@ def _ulp_close(got, want_f32, dtype):
 
 # ------------------------------------------------------------------------------------ pooling
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
-@pytest.mark.parametrize("n,block,d", [(256, 64, 64), (200, 64, 64), (1041, 64, 64), (96, 16, 64), (130, 32, 32), (7, 64, 64)])
+@pytest.mark.parametrize("n,block,d", [(256, 64, 64), (200, 64, 64), (1041, 64, 64), (96, 16, 64), (130, 32, 32), (7, 64, 64),
+                                       (1041, 16, 64), (1000, 8, 64), (333, 32, 64), (5, 16, 64), (64, 16, 64), (200, 4, 64)])
 def test_pool_matches_oracle(dtype, n, block, d):
     x = _randn((2, 3, n, d), n + d, dtype)
     got = s3r.pool_mean(x.to(DEV), block)
