@@ -262,6 +262,8 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     // threshold = score of the list's last entry (key 0, a filler, maps to a NaN, which fmaxf drops: thr0 remains)
     const uint32_t k32 = key_sortable(list[KL - 1]);
     thr = fmaxf(__uint_as_float(k32 ^ ((k32 & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)), thr0);  // fmaxf drops the NaN
+    // the partner lane's bound holds for this lane too: K keys of the same query row score at least that much
+    thr = fmaxf(thr, __uint_as_float(xh_swap(__float_as_uint(thr))));
   };
 
   const int ntiles = (int)((Lk + 63) / 64);
@@ -424,15 +426,17 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     };
     const uint32_t lds_k = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(&Ks[0][0]);
     const uint32_t kr_off = lds_k + (uint32_t)(c * 128 + ((hh ^ (c & 7)) << 4));  // A operand: lane = key row, chunk hh + 2 ks
-    auto sweep = [&](auto filter_tag) {
+    auto sweep = [&](auto filter_tag, const int stride) {  // tiles 0, stride, 2 stride, ...
       constexpr bool FILTER = decltype(filter_tag)::value;
-      for (int i = 0; i < NB - 1; i++) dma_tile(i, i);
-      int buf = 0, fill = NB - 1;  // ring positions of tile t and of tile t + NB - 1
-      for (int t = 0; t < ntiles; t++) {
+      const int nsteps = (ntiles + stride - 1) / stride;
+      for (int i = 0; i < NB - 1; i++) dma_tile(i * stride, i);
+      int buf = 0, fill = NB - 1;  // ring positions of step i's tile and of step i + NB - 1's
+      for (int i = 0; i < nsteps; i++) {
+        const int t = i * stride;
         // this wave's share of tile t has landed (transfers complete in order, two per tile, NB - 2 tiles younger) ...
         __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NB - 2)));
         __builtin_amdgcn_s_barrier();  // ... and everybody's; all waves are done with tile t - 1, whose buffer is refilled now
-        dma_tile(t + NB - 1, fill);
+        dma_tile((i + NB - 1) * stride, fill);
         {
           const int64_t start = (int64_t)t * 64;
           const bool partial = start + 64 > Lk;
@@ -498,6 +502,9 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
                 // Branch-free append, five VALU instructions: survivors (score >= thr; thr is never a NaN, a masked
                 // key's NaN fails) go to queue slot qn, the others to the dump slot; every lane writes (score, column).
                 uint32_t slot, col;
+                // survivors are a fraction of a percent of the scores: most of the time none of the 64 lanes has one at
+                // this register, and the whole append is skipped for one compare and a scalar branch
+                if (__builtin_expect(__builtin_amdgcn_ballot_w64(st[kt][r] >= thr) == 0, 1)) continue;
                 asm volatile(
                     "v_cmp_ge_f32 vcc, %[s], %[thr]\n\t"
                     "v_cndmask_b32 %[slot], %[dump], %[qn], vcc\n\t"
@@ -517,7 +524,11 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the transfers issued past the last tile are done too
     };
     // First sweep: every lane keeps the K largest of its half-tile maxima (maxima over 32 different keys each).
-    sweep(std::false_type{});
+    // A sample of the tiles is enough: the K-th largest maximum over any subset of the keys is still a lower bound.
+    // With fewer sampled tiles the bound is looser (more survivors in the second sweep) but the sweep shorter;
+    // about 32 sampled tiles balance the two (measured at 66 and 261 tiles).
+    const int stride1 = ntiles >= 64 ? (ntiles / 32 < 8 ? ntiles / 32 : 8) : 1;
+    sweep(std::false_type{}, stride1);
     // Threshold: the K-th largest of the row's half-tile maxima, i.e. of the union of the two lanes' lists.  K
     // different scores (one per half tile) are at least that large, so a score below it is not among the K
     // largest, whatever the tie-break.  With fewer than K half tiles it stays -inf and every score is a candidate.
@@ -535,7 +546,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     // Second sweep: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
     // through the lane's queue into its exact list.
     __syncthreads();  // every wave is done with the tile buffers of the first sweep
-    sweep(std::true_type{});
+    sweep(std::true_type{}, 1);
     drain();
     // the K best of this lane's list and the partner lane's, descending: max of entry i with the partner's entry
     // K-1-i (a bitonic sequence), two entries at a time so that no second copy of the list is held, then one merge
