@@ -154,16 +154,23 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
     for (int r = 0; r < 16; r++) st[r] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) st = Mma<E>::mma(ak[ks], bq[QT][ks], st);
-    // register r holds key row 4hh + 8(r/4) + r%4 of the half tile: rows 0-15 (r < 8) are block 0's keys, 16-31 block 1's
-    float mx = -INFINITY;
+    // register r holds key row 4hh + 8(r/4) + r%4 of the half tile: rows 0-15 (r < 8) are block 0's keys, 16-31 block
+    // 1's.  Only the 8 registers of this lane's own block are scores of its query: they are picked first, and the
+    // softmax runs on 8 values instead of 16.
+    const uint32_t m0 = mine == 0 ? 0xFFFFFFFFu : 0u;  // bit masks instead of per-value selects on a condition register
+    const uint32_t own_sel = mine == 0 ? 0x07060504u : 0x03020100u;  // v_perm_b32 selector: all four bytes of the first / second source
+    float su[8];
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int krow_in_blk = 4 * hh + 8 * ((r >> 2) & 1) + (r & 3);
-      const bool ok = ((r >> 3) == mine) && (krow_in_blk < nkeys);
-      st[r] = ok ? st[r] * sl2 : -INFINITY;
-      mx = fmaxf(mx, st[r]);
+    for (int j = 0; j < 8; j++) su[j] = __uint_as_float(__builtin_amdgcn_perm(__float_as_uint(st[j]), __float_as_uint(st[8 + j]), own_sel));
+    if (__any(nkeys < 16)) {  // a ragged last block or a skipped entry somewhere in the wave
+#pragma unroll
+      for (int j = 0; j < 8; j++)
+        if (4 * hh + 8 * (j >> 2) + (j & 3) >= nkeys) su[j] = -INFINITY;
     }
-    mx = xh_max(mx);
+    float mx = su[0];
+#pragma unroll
+    for (int j = 1; j < 8; j++) mx = fmaxf(mx, su[j]);
+    mx = xh_max(mx) * sl2;  // sl2 > 0: the maximum of the scaled scores
     const float m_new = fmaxf(m_i[QT], mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;   // nothing valid so far: every probability is exp2(-inf) = 0
     const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - m_use);  // 0 while m_i is -inf
@@ -175,18 +182,23 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
         for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
     }
     m_i[QT] = m_new;
-    V8 pf[2];
+    // probabilities of the own block, then the B operand of the PV product: the own block's k-group carries them,
+    // the other block's k-group zeros
+    union { V8 v; uint32_t w[4]; } pown, pf[2];
 #pragma unroll
-    for (int jj = 0; jj < 2; jj++)
+    for (int e = 0; e < 8; e += 2) {
+      V2 pk;
+      pk[0] = (E)__builtin_amdgcn_exp2f(fmaf(su[e], sl2, -m_use));
+      pk[1] = (E)__builtin_amdgcn_exp2f(fmaf(su[e + 1], sl2, -m_use));
+      pown.v[e] = pk[0];
+      pown.v[e + 1] = pk[1];
+      l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
+    }
 #pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        V2 pk;
-        pk[0] = (E)__builtin_amdgcn_exp2f(st[8 * jj + e] - m_use);
-        pk[1] = (E)__builtin_amdgcn_exp2f(st[8 * jj + e + 1] - m_use);
-        pf[jj][e] = pk[0];
-        pf[jj][e + 1] = pk[1];
-        l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
-      }
+    for (int wi = 0; wi < 4; wi++) {
+      pf[0].w[wi] = pown.w[wi] & m0;
+      pf[1].w[wi] = pown.w[wi] & ~m0;
+    }
     V8 vfr[2][2];
 #pragma unroll
     for (int jj = 0; jj < 2; jj++)
@@ -201,7 +213,7 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
 #pragma unroll
     for (int jj = 0; jj < 2; jj++)
 #pragma unroll
-      for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[jj], ot[dt][QT]);
+      for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[jj].v, ot[dt][QT]);
   };
 
   const int nsteps = p.K;
