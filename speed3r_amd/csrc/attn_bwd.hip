@@ -58,8 +58,9 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const E* __restrict__ o,
   const int64_t n = rr % N, bh = rr / N;
   const int h = (int)(bh % H);
   const int64_t b = bh / H;
-  const uint4 a = *reinterpret_cast<const uint4*>(o + b * sob + h * soh + n * son + part * 8);
-  const uint4 g = *reinterpret_cast<const uint4*>(dout + b * sdb + h * sdh + n * sdn + part * 8);
+  // both tensors are streamed once: non-temporal loads
+  const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(o + b * sob + h * soh + n * son + part * 8));
+  const u32x4 g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dout + b * sdb + h * sdh + n * sdn + part * 8));
   const E* ae = reinterpret_cast<const E*>(&a);
   const E* ge = reinterpret_cast<const E*>(&g);
   float s = 0.f;

@@ -98,7 +98,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         int row = 32 * qt + 8 * i + qr;
         row = row < q_last ? row : q_last;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16,
-                                                 (uint32_t)row * q_rowbytes + q_chunk, 0, 0, 0);
+                                                 (uint32_t)row * q_rowbytes + q_chunk, 0, 0, 2 /* nt: the Q block is read once */);
       }
     }
   }
