@@ -73,11 +73,13 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const E* __restrict__ o,
 
 // ---- shared pieces of the two MFMA kernels -----------------------------------------------------------------------
 // Transfer of rows [8*i0*.., ...) of a 32-row half tile: instruction i moves rows 8i .. 8i+7 (16 bytes per lane).
-// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ tsw(row), tsw = 4*bit1(row) | 2*bit2(row): bit 2 of the chunk
-// spreads the four rows of a transposed read over disjoint bank groups, bit 1 separates rows r and r+4 for the
-// 16-byte row reads, so both kinds of read are conflict free on the same buffer.  Otherwise c' ^ (row&7) (row reads
-// only).  Rows are clamped to `last` (relative to `base`'s row 0).
-__device__ __forceinline__ int tsw(int row) { return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1); }
+// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ tsw(row), tsw(row) = bit2 | (bit0 ^ bit1) << 1 | bit1 << 2 of the
+// row: of the 32768 GF(2)-linear maps from the 5 row bits to the 3 chunk bits, timed on the device, this is one of
+// those whose 16-byte row reads AND ds_read_b64_tr_b16 reads both run without bank conflicts (the transposed reads
+// take 1.3x as long with the plain (row & 7) map or none), and it only looks at row bits 0..2, so rows 8 and 16
+// further down keep the same map.  Otherwise c' ^ (row & 7) (row reads only).  Rows are clamped to `last`
+// (relative to `base`'s row 0).
+__device__ __forceinline__ int tsw(int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ row) & 1) << 1) | (((row >> 1) & 1) << 2); }
 
 template <typename E, bool VSW>
 __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int first_row, int last, char* lds_half, int lane, int i_begin, int i_end) {
