@@ -36,6 +36,8 @@ def parse_args():
                     help="cfg1-cfg4: one sparse global-attention layer call; cfg5: end-to-end Pi3_Sparse-style forward (frames/s)")
     ap.add_argument("--frames", type=int, default=100, help="cfg5: number of 518x392 frames")
     ap.add_argument("--topk", type=int, default=None)
+    ap.add_argument("--block", type=int, default=64, choices=[16, 64],
+                    help="tokens per block: 64 (the headline workload) or 16 (the reference layer's own block size, with --topk 32)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
@@ -174,7 +176,7 @@ def run_backward(args, cfg, qd, kd, vd, block, topk) -> int:
         wall = time.perf_counter() - t0
     ms = wall * 1e3 / args.steps
     kern = {nm: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i, nm in enumerate(names)}
-    mm = workloads.selection_flops(n, topk) / 2          # one product over the selected (query block, key block) pairs
+    mm = workloads.selection_flops(n, topk, block=block) / 2          # one product over the selected (query block, key block) pairs
     f_dq, f_dkdv = 3 * mm, 4 * mm
     dom = "dkdv" if kern["dkdv"] >= kern["dq"] else "dq"
     tfl = (f_dkdv if dom == "dkdv" else f_dq) / (kern[dom] * 1e-3) / 1e12
@@ -184,7 +186,7 @@ def run_backward(args, cfg, qd, kd, vd, block, topk) -> int:
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{cfg.name} backward: {n} tokens, 16 heads x 64, block {block}, top-k {topk}, B=1"},
         "kernels_ms": kern,
-        "effective_tflops": (f_dq + f_dkdv + 2.5 * workloads.compressed_flops(n)) / (ms * 1e-3) / 1e12,
+        "effective_tflops": (f_dq + f_dkdv + 2.5 * workloads.compressed_flops(n, block=block)) / (ms * 1e-3) / 1e12,
         "roofline": {"kernel": "bwd_dkdv_kernel" if dom == "dkdv" else "bwd_dq_kernel", "bound": "mfma", "achieved": tfl,
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS, "traffic": None},
     }))
@@ -209,7 +211,7 @@ def main() -> int:
     dev = torch.device("cuda:0")
     cfg, q, k, v, gate = workloads.make_config(args.config)
     topk = args.topk or cfg.topk
-    block = workloads.BLOCK
+    block = args.block
     n = cfg.tokens
     qd, kd, vd, gd = (t.to(dev) for t in (q, k, v, gate))
     mat = True if args.materialize_scores else None
@@ -264,6 +266,7 @@ def main() -> int:
     def span(a, b):
         return sum(e[a].elapsed_time(e[b]) for e in evs) / args.steps
 
+    fused = fused and "merge" not in evs[0]   # the merge runs in the selection kernel's epilogue only where that is built
     sel_name = "select_merge" if fused else "select"
     if overlap:   # the index kernel runs on a second stream beside the pooling of v and the compressed attention
         kern_ms = {"pool+compressed_topk (two streams)": span("start", "select")}
@@ -274,8 +277,8 @@ def main() -> int:
     else:
         kern_ms["select"] = span("select", "merge")
         kern_ms["merge"] = span("merge", "end")
-    f_sel = workloads.selection_flops(n, topk)
-    f_cmp = workloads.compressed_flops(n)
+    f_sel = workloads.selection_flops(n, topk, block=block)
+    f_cmp = workloads.compressed_flops(n, block=block)
     sel_tflops = f_sel / (kern_ms[sel_name] * 1e-3) / 1e12
     es = 2 if cfg.dtype != torch.float32 else 4
     pool_bytes = 3 * (n + nc) * 16 * 64 * es
@@ -306,7 +309,7 @@ def main() -> int:
                     **({} if fused else {"merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9})},
         "peak_mem_gb": peak_mem / 1e9,
         "roofline": {
-            "kernel": "select_pipe_kernel" + (" (gated merge in its epilogue)" if fused else ""),
+            "kernel": ("select_pipe_kernel" if block == 64 else "select_b16_kernel") + (" (gated merge in its epilogue)" if fused else ""),
             "bound": "mfma",
             "achieved": sel_tflops,
             "peak": PEAK_BF16_TFLOPS,
@@ -314,7 +317,7 @@ def main() -> int:
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
             # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a plain copy (profiles/); measured for the
             # default workload only
-            "traffic": 2.41e9 if (fused and args.config == "cfg3" and topk == 16) else None,
+            "traffic": 2.41e9 if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
         },
     }
     if not args.no_cpu_baseline:
