@@ -121,7 +121,7 @@ int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* 
  * Replaces topk_blocksparse_attention (pi3/models/sparse_attn/topk_blocksparse_attention.py:1093-1121)
  * together with the merge expression of pi3/models/layers/sparse_attention.py:127-136.
  * Arguments as in s3r_select_attn and s3r_gated_merge; out is contiguous [B,N,H*D].
- * Only for the MFMA path (bf16/fp16, D == 64, block == 64, 16-byte aligned tensors); other
+ * Only for the MFMA paths (bf16/fp16, D == 64, block == 64 or 16, 16-byte aligned tensors); other
  * shapes return S3R_ERR_UNSUPPORTED and the caller runs the two operators one after the other.
  */
 int s3r_select_attn_merge(const void* q, const void* k, const void* v, const int32_t* idx,

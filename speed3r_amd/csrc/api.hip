@@ -109,17 +109,19 @@ static int select_attn_impl(const char* who, const void* q, const void* k, const
     const char* e = getenv("S3R_SELECT_KERNEL");
     return e != nullptr && strcmp(e, "basic") == 0;
   }();
+  // 16-token blocks (the reference layer's own setting): MFMA kernel that pairs query blocks
+  const bool b16_ok = dtype != S3R_F32 && D == 64 && block == 16 && K <= 64 && softmax_scale > 0.f &&
+                      skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
+                      vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
+                      (merge ? (vec_ok(m.o_cmp, es, m.scb, m.sch, m.scm) && aligned16(m.out)) : vec_ok(o, es, sob, soh, son));
   if (merge) {
+    if (b16_ok) return launch_select_b16(p, dtype, stream);
     if (!mfma_ok || basic)
-      return fail(S3R_ERR_UNSUPPORTED, "%s: the fused merge needs the pipelined MFMA kernel (bf16/fp16, head_dim 64, block 64, "
+      return fail(S3R_ERR_UNSUPPORTED, "%s: the fused merge needs an MFMA kernel (bf16/fp16, head_dim 64, block 64 or 16, "
                                        "16-byte aligned tensors); run s3r_select_attn and s3r_gated_merge instead", who);
     return launch_select_pipe(p, dtype, stream);
   }
   if (mfma_ok) return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
-  // 16-token blocks (the reference layer's own setting): MFMA kernel that pairs query blocks
-  const bool b16_ok = dtype != S3R_F32 && D == 64 && block == 16 && K <= 64 && softmax_scale > 0.f &&
-                      skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
-                      vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) && vec_ok(o, es, sob, soh, son);
   if (b16_ok) return launch_select_b16(p, dtype, stream);
   return launch_attn_simple(p, dtype, /*select=*/true, stream);
 }

@@ -235,13 +235,24 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
     }
   }
 
-  // output: as in the 64-token kernels (one exchange with lane ^ 32 per packed word, 16-byte stores)
+  // output: as in the 64-token kernels (one exchange with lane ^ 32 per packed word, 16-byte stores).  With merge
+  // operands the gated merge runs here (gate pair of the row, the compressed output of the row's 16-token block; the
+  // three roundings of the eager expression kept) and the result goes to the [B, N, H*D] tensor.
+  const bool merge = p.merge_out != nullptr;
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
     const float l = xh_sum(l_i[qt]);
     const float inv = l > 0.f ? 1.f / l : 0.f;
     const int64_t row = q0 + qt * 32 + c;
     const bool live = row < N;
+    float g0 = 0.f, g1 = 0.f;
+    const E* ocp = nullptr;
+    if (merge && live) {
+      const E* gp = (const E*)p.merge_gate + (int64_t)b * p.sgb + (int64_t)h * p.sgh + row * p.sgn;
+      g0 = (float)gp[0];
+      g1 = (float)gp[1];
+      ocp = (const E*)p.merge_oc + (int64_t)b * p.scb + (int64_t)h * p.sch + (row >> 4) * p.scm;
+    }
 #pragma unroll
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -260,7 +271,22 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
           pc.w[wi] = r[0];
           pc.w[2 + wi] = r[1];
         }
-        if (live) *reinterpret_cast<uint4*>(op + row * p.som + dt * 32 + 8 * (2 * gp + hh)) = pc.u;
+        const int d0 = dt * 32 + 8 * (2 * gp + hh);
+        if (live) {
+          if (!merge) {
+            *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
+          } else {
+            union { E e[8]; uint4 u; } oc, res;
+            oc.u = *reinterpret_cast<const uint4*>(ocp + d0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const float x = round_to<E>(g0 * (float)oc.e[e]);
+              const float y = round_to<E>(g1 * (float)pc.e[e]);
+              res.e[e] = (E)(x + y);
+            }
+            *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = res.u;
+          }
+        }
       }
     if (live && p.lse != nullptr && hh == 0)
       p.lse[((int64_t)b * p.H + h) * N + row] = l > 0.f ? (m_i[qt] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;

@@ -262,7 +262,7 @@ def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: to
     assert idx.shape[:3] == (b, h, nqb), f"topk_idx shape {tuple(idx.shape)} does not match {(b, h, nqb, 'K')}"
     assert o_cmp.shape == (b, h, nqb, d), f"o_cmp shape {tuple(o_cmp.shape)} != {(b, h, nqb, d)}"
     assert gate.shape == (b, h, n, 2), f"gate shape {tuple(gate.shape)} != {(b, h, n, 2)}"
-    if q.dtype == torch.float32 or d != 64 or block != 64 or idx.shape[3] > 64:
+    if q.dtype == torch.float32 or d != 64 or block not in (64, 16) or idx.shape[3] > 64:
         return None
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
     out = torch.empty((b, n, h * d), dtype=q.dtype, device=q.device)

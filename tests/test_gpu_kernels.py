@@ -232,11 +232,12 @@ def test_select_fixture(golden):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("n,h,kk", [(256, 2, 2), (200, 3, 4), (1041, 2, 16), (64, 1, 1)])
-def test_select_with_fused_merge_equals_the_two_operators(dtype, n, h, kk):
+@pytest.mark.parametrize("n,h,kk,block", [(256, 2, 2, 64), (200, 3, 4, 64), (1041, 2, 16, 64), (64, 1, 1, 64),
+                                          (256, 2, 4, 16), (200, 3, 8, 16), (1041, 2, 32, 16), (40, 1, 1, 16)])
+def test_select_with_fused_merge_equals_the_two_operators(dtype, n, h, kk, block):
     """The merge in the selection kernel's epilogue must give the bits of select_attn followed by gated_merge
     (ragged tail, skipped entries and empty rows included) and agree with the oracle's merge of the oracle's selection."""
-    b, d, block = 2, 64, 64
+    b, d = 2, 64
     nqb = -(-n // block)
     q, k, v = (_randn((b, h, n, d), 20 + i, dtype, 0.5).to(DEV) for i in range(3))
     g = torch.Generator().manual_seed(5)
@@ -256,7 +257,7 @@ def test_select_with_fused_merge_equals_the_two_operators(dtype, n, h, kk):
 
 
 def test_fused_merge_declines_shapes_without_an_mfma_kernel():
-    b, h, n, d, block = 1, 2, 96, 64, 16
+    b, h, n, d, block = 1, 2, 96, 64, 32
     q, k, v = (_randn((b, h, n, d), 40 + i, torch.bfloat16).to(DEV) for i in range(3))
     idx = torch.zeros((b, h, n // block, 2), dtype=torch.int32, device=DEV)
     o_cmp = _randn((b, h, n // block, d), 43, torch.bfloat16).to(DEV)
