@@ -37,14 +37,18 @@ constexpr int kWaves = S3R_PIPE_WAVES;  // wavefronts (= query blocks) per workg
 
 // DENSE: no index list, every query block attends to all key tiles in order (the compressed branch's attention over
 // the pooled tokens runs through this instance).
-template <typename E, bool DENSE>
+// SPLIT (with DENSE, for sweeps with too few query blocks to fill the chip): two waves share a query block, each
+// sweeps half of the key tiles, and the first one folds the second one's accumulators into its own through LDS.
+template <typename E, bool DENSE, bool SPLIT = false>
 __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
+  static_assert(!SPLIT || DENSE, "the split sweep is a variant of the dense one");
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[kWaves * kHalf * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[kWaves * kHalf * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kWaves * kHalf * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kWaves * kHalf * 2];
+  __shared__ float lds_ml[SPLIT ? kWaves * 4 * 64 : 1];  // SPLIT: per wave and lane the two references and the two row sums
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int lane = threadIdx.x & 63;
@@ -59,7 +63,12 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const int qg = vid - bh * nqg;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
-  const int qb = qg * kWaves + wave;
+  const int split = SPLIT ? (wave & 1) : 0;  // which half of the key tiles
+  int qb = SPLIT ? qg * (kWaves / 2) + (wave >> 1) : qg * kWaves + wave;
+  // SPLIT: every wave of the workgroup has to reach the barrier of the hand-over, so a pair past the last query block
+  // repeats the last block's work and stores nothing
+  const bool ghost = SPLIT && qb >= nqb;
+  if (SPLIT) qb = qb < nqb ? qb : nqb - 1;
   if (qb >= nqb) return;
 
   const int64_t N = p.Lq;
@@ -109,10 +118,19 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   bool my_valid = false;
   uint64_t todo = 0;
   int n_ragged, n_full;
-  int dense_next = 0;  // DENSE: the next tile of the sweep
+  int dense_next = 0;  // DENSE: the next tile of the sweep and the end of this wave's range
+  int dense_begin = 0, dense_end = 0;
   if constexpr (DENSE) {
     n_full = (int)(N >> 6);
     n_ragged = (N & 63) ? 1 : 0;
+    if constexpr (SPLIT) {  // first wave: tiles [0, h0); second wave: [h0, n_full) and the ragged tile
+      const int h0 = (n_full + 1) >> 1;
+      dense_begin = split ? h0 : 0;
+      n_full = split ? n_full - h0 : h0;
+      n_ragged = split ? n_ragged : 0;
+    }
+    dense_next = dense_begin;
+    dense_end = dense_begin + n_full;
   } else {
     // The list comes through the scalar cache (s_load): a vector load would wait in the vector memory queue behind
     // the Q transfers and behind the other waves' tile transfers, and the first K transfer waits for the list.
@@ -140,7 +158,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
     n_full = __popcll(todo);
   }
-  if (n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
+  if (!SPLIT && n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer may still write LDS when the wave ends
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
@@ -460,7 +478,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     int64_t last_start = 0;
     auto pop_or_last = [&]() -> int64_t {  // branch-free: next full tile, or the last one again
       if constexpr (DENSE) {
-        last_start = (int64_t)(dense_next < n_full ? dense_next : n_full - 1) * 64;
+        last_start = (int64_t)(dense_next < dense_end ? dense_next : dense_end - 1) * 64;
         dense_next++;
         return last_start;
       }
@@ -519,7 +537,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   if (redo) {  // rare: recompute the query block with the online softmax
     reset_state();
     if constexpr (DENSE) {
-      for (int t = 0; t < n_full; t++) robust_tile((int64_t)t * 64);
+      for (int t = dense_begin; t < dense_end; t++) robust_tile((int64_t)t * 64);
     } else {
       uint64_t again = __ballot(my_valid && my_idx != ragged_blk);
       while (again) {
@@ -534,6 +552,43 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   // Output: lane (c, hh) holds for query c + 32*qt the head_dim values dt*32 + 8*g4 + 4*hh + {0..3}.  One exchange with
   // lane ^ 32 per packed word hands every lane eight consecutive head_dim values (hh = 0: group g4 = 2*gp, hh = 1:
   // group 2*gp + 1), so a row receives 32 contiguous bytes per store instruction.
+  if constexpr (SPLIT) {
+    // the second wave of a pair hands its state over: accumulators [dt][qt] into its four (now idle) 4 KB buffers,
+    // register r of lane l at float r*64 + l, references and row sums into lds_ml; the first wave folds them in
+    auto xo = [&](int w, int dt, int qt) -> float* {
+      unsigned char* a = dt == 0 ? (qt == 0 ? lds_k0 : lds_k1) : (qt == 0 ? lds_v0 : lds_v1);
+      return reinterpret_cast<float*>(a + w * (kHalf * 2));
+    };
+    if (split == 1) {
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) xo(wave, dt, qt)[r * 64 + lane] = ot[dt][qt][r];
+#pragma unroll
+      for (int qt = 0; qt < 2; qt++) {
+        lds_ml[(wave * 4 + qt) * 64 + lane] = m_i[qt];
+        lds_ml[(wave * 4 + 2 + qt) * 64 + lane] = l_i[qt];
+      }
+    }
+    __syncthreads();
+    if (split == 1 || ghost) return;
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      const float m1 = lds_ml[((wave + 1) * 4 + qt) * 64 + lane];
+      const float l1 = lds_ml[((wave + 1) * 4 + 2 + qt) * 64 + lane];
+      const float mt = fmaxf(m_i[qt], m1);
+      const float a0 = mt == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_i[qt] - mt);  // exp2(-inf) = 0 for an empty half
+      const float a1 = mt == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mt);
+      l_i[qt] = l_i[qt] * a0 + l1 * a1;
+      m_i[qt] = mt;
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) ot[dt][qt][r] = ot[dt][qt][r] * a0 + xo(wave + 1, dt, qt)[r * 64 + lane] * a1;
+    }
+  }
   if (!merge_loaded) load_merge_operands();
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
@@ -587,20 +642,25 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
 
 int launch_select_pipe(const AttnParams& p, int dtype, void* stream) {
   const int64_t nqb = (p.Lq + 63) / 64;
-  const int64_t nqg = (nqb + pipe::kWaves - 1) / pipe::kWaves;
+  const bool dense = p.idx == nullptr;  // no index list: every query block sweeps all key tiles
+  if (dense && p.Lq != p.Lk) return fail(S3R_ERR_UNSUPPORTED, "dense sweep: Lq %lld != Lk %lld", (long long)p.Lq, (long long)p.Lk);
+  // a dense sweep with fewer waves than 1.5 per SIMD of the chip (256 CUs x 4) runs with two waves per query block
+  const bool split = dense && nqb * p.B * p.H < 1536;
+  const int per_wg = split ? pipe::kWaves / 2 : pipe::kWaves;
+  const int64_t nqg = (nqb + per_wg - 1) / per_wg;
   const int64_t total = nqg * p.B * p.H;
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)total), blk(64 * pipe::kWaves);
-  const bool dense = p.idx == nullptr;  // no index list: every query block sweeps all key tiles
-  if (dense && p.Lq != p.Lk) return fail(S3R_ERR_UNSUPPORTED, "dense sweep: Lq %lld != Lk %lld", (long long)p.Lq, (long long)p.Lk);
-  if (dtype == S3R_BF16) {
-    if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<bf16_t, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
-    else hipLaunchKernelGGL((pipe::select_pipe_kernel<bf16_t, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
-  } else {
-    if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<f16_t, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
-    else hipLaunchKernelGGL((pipe::select_pipe_kernel<f16_t, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);
-  }
+#define S3R_PIPE_LAUNCH(E)                                                                                                       \
+  do {                                                                                                                           \
+    if (split) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total); \
+    else if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);  \
+    else hipLaunchKernelGGL((pipe::select_pipe_kernel<E, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);            \
+  } while (0)
+  if (dtype == S3R_BF16) S3R_PIPE_LAUNCH(bf16_t);
+  else S3R_PIPE_LAUNCH(f16_t);
+#undef S3R_PIPE_LAUNCH
   return check_launch("select_pipe_kernel");
 }
 

@@ -117,6 +117,23 @@ def test_compressed_matches_oracle(dtype, lq, lk):
     np.testing.assert_array_equal(idx.cpu().numpy(), oracle.topk_from_scores(scores.cpu(), k))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("h,n", [(3, 1), (3, 63), (2, 64), (3, 65), (2, 128), (3, 129), (2, 200), (3, 1041), (16, 4164), (24, 4096)])
+def test_dense_sweep_of_the_pipelined_kernel_matches_oracle(dtype, h, n):
+    """The attention of the compressed branch without a score buffer runs as a dense sweep of the selection kernel:
+    with few query blocks two waves share a block and sweep half of the key tiles each (every case here but the
+    last), otherwise one wave sweeps them all (24 heads x 64 blocks).  One to 66 tiles, ragged last tiles, odd and
+    even tile counts, a last workgroup with a single pair."""
+    q = _randn((1, h, n, 64), n, dtype, 0.5)
+    k = _randn((1, h, n, 64), n + 1, dtype, 0.5)
+    v = _randn((1, h, n, 64), n + 2, dtype)
+    o, idx, lse = s3r.compressed_attn_topk(q.to(DEV), k.to(DEV), v.to(DEV), None, return_lse=True)
+    assert idx is None
+    o_ref, lse_ref, _ = oracle.compressed_attention(q, k, v, out_dtype=torch.float32)
+    assert max_abs(o, o_ref) <= TOL[dtype]
+    assert max_abs(lse, lse_ref) <= 2e-3
+
+
 def test_compressed_fixture(golden):
     qc, kc, vc = (from_bf16_bits(golden[n]) for n in ("qc", "kc", "vc"))
     o, idx, scores = s3r.compressed_attn_topk(qc.to(DEV), kc.to(DEV), vc.to(DEV), 8, return_scores=True)
