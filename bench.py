@@ -317,7 +317,7 @@ def main() -> int:
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
             # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a plain copy (profiles/); measured for the
             # default workload only
-            "traffic": 2.41e9 if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
+            "traffic": 2.34e9 if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
         },
     }
     if not args.no_cpu_baseline:
