@@ -343,7 +343,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         pk[1] = (E)x1;
         pf[qt][KT][jj][e8] = pk[0];
         pf[qt][KT][jj][e8 + 1] = pk[1];
-        l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
+        l_i[qt] += x0;  // row sums over the unrounded probabilities, as the reference's tl.sum(p) before p.to(v.dtype)
+        l_i[qt] += x1;
         asm volatile("" : "+v"(pf[qt][KT][jj]), "+v"(l_i[qt]));
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -405,12 +406,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         for (int jj = 0; jj < 2; jj++)
 #pragma unroll
           for (int e = 0; e < 8; e += 2) {
-            V2 pk;
-            pk[0] = (E)__builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e], sl2, -m_new));
-            pk[1] = (E)__builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e + 1], sl2, -m_new));
-            pf[qt][kt][jj][e] = pk[0];
-            pf[qt][kt][jj][e + 1] = pk[1];
-            l_i[qt] = Mma<E>::dot_ones(pk, l_i[qt]);
+            const float x0 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e], sl2, -m_new));
+            const float x1 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e + 1], sl2, -m_new));
+            pf[qt][kt][jj][e] = (E)x0;
+            pf[qt][kt][jj][e + 1] = (E)x1;
+            l_i[qt] += x0 + x1;
           }
     }
     read_v(H0{}, vfr);
