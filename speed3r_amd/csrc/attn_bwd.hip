@@ -27,11 +27,13 @@
 // never read (transfers re-read the last valid row).
 //
 // 16-token blocks (BLK = 16, the reference layer's own block size) run through the same kernels: a 32-row half tile
-// is then two 16-row blocks taken from two different lists (query blocks 2h, 2h+1 of the wave's 64 queries and entry t
-// of each one's index list in the dQ kernel; key blocks 2w, 2w+1 of the tile and entry t of each one's query-block
-// list in the dK/dV kernel).  A 32 x 32 product holds the two wanted 16 x 16 blocks on its diagonal; the other two
-// quadrants get P = 0.  Half h of the keys only meets half h of the queries, so the other half's products are not
-// issued at all.
+// is then two 16-row blocks.  dQ kernel: query blocks 2h, 2h+1 of the wave's 64 queries and entry t of each one's
+// index list; key half h only meets query half h, so the other half's products are not issued.  dK/dV kernel: a wave
+// takes one 16-key block at a time, held twice (lanes c and c + 16 carry key c & 15), against entries 2t and 2t + 1 of
+// that block's query-block list, and adds the two halves' partial sums when the list ends.  Either way the wanted
+// 16 x 16 blocks sit on the diagonal of a 32 x 32 product and the other two quadrants get P = 0.  Tiles whose lists
+// are long (first pass of the grid) share every list between the workgroup's two waves, which hand partial sums over
+// through LDS; the other tiles give each wave two key blocks of its own.
 #include "select_common.h"
 #include "attn_bwd.h"
 
@@ -433,10 +435,10 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     int len;
     if constexpr (BLK == 64) {
       len = off[kb + 1] - off[kb];
-    } else {  // the longer of this wave's two lists (the waves of a workgroup are independent)
-      const int64_t ka = (int64_t)kb * 4 + 2 * wave;
-      const int la = ka < nkbl ? off[ka + 1] - off[ka] : 0, lb = ka + 1 < nkbl ? off[ka + 2] - off[ka + 1] : 0;
-      len = la > lb ? la : lb;
+    } else {  // the workgroup walks the lists of its four key blocks one after the other, four entries per step
+      const int64_t ka = (int64_t)kb * 4;
+      const int64_t kz = ka + 4 < nkbl ? ka + 4 : nkbl;
+      len = (off[kz] - off[ka]) / 4;
     }
     len = __builtin_amdgcn_readfirstlane(len);
     if ((len > 4 * p.K) != long_pass) return;
@@ -448,33 +450,38 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
   const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
 
-  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks)
-  const int64_t key = (int64_t)kb * 64 + wave * 32 + c;
+  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks).  BLK 16: the wave takes its two
+  // key blocks one after the other, and lanes c and c + 16 both hold key c & 15 of the current block: each half of
+  // the lanes then meets its own 16-query block of the tile (two list entries per step), and the two halves' partial
+  // dK^T, dV^T are added up when the list ends.
+  int64_t key = (int64_t)kb * 64 + wave * 32 + c;
   V8 bk[4], bv[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ks++) {
-    Frag f, g;
-    f.u = make_uint4(0, 0, 0, 0);
-    g.u = make_uint4(0, 0, 0, 0);
-    if (key < Lk) {
-      f.u = *reinterpret_cast<const uint4*>(kp + key * p.skn + ks * 16 + hh * 8);
-      g.u = *reinterpret_cast<const uint4*>(vp + key * p.svn + ks * 16 + hh * 8);
-    }
-    bk[ks] = as_v8<E>(f);
-    bv[ks] = as_v8<E>(g);
-  }
   f32x16 dkt[2], dvt[2];  // dK^T, dV^T [dt]: lane = key, registers = head_dim
+  auto load_keys = [&]() {
 #pragma unroll
-  for (int dt = 0; dt < 2; dt++)
+    for (int ks = 0; ks < 4; ks++) {
+      Frag f, g;
+      f.u = make_uint4(0, 0, 0, 0);
+      g.u = make_uint4(0, 0, 0, 0);
+      if (key < Lk) {
+        f.u = *reinterpret_cast<const uint4*>(kp + key * p.skn + ks * 16 + hh * 8);
+        g.u = *reinterpret_cast<const uint4*>(vp + key * p.svn + ks * 16 + hh * 8);
+      }
+      bk[ks] = as_v8<E>(f);
+      bv[ks] = as_v8<E>(g);
+    }
 #pragma unroll
-    for (int r = 0; r < 16; r++) { dkt[dt][r] = 0.f; dvt[dt][r] = 0.f; }
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) { dkt[dt][r] = 0.f; dvt[dt][r] = 0.f; }
+  };
+  if constexpr (BLK == 64) load_keys();
 
   // query blocks that attend to this key block
   static_assert(BLK == 64 || (BLK == 16 && !DENSE), "blocks of 64 tokens, or of 16 with key-centric lists");
   int n_lists;
   const int32_t* list = nullptr;
-  const int32_t* list_b = nullptr;  // BLK 16: `list` belongs to this wave's first key block (2w of the tile), list_b to its second
-  int len_a = 0, len_b = 0;
+  const int32_t* off16 = nullptr;  // BLK 16: the list offsets of this (b, h); `list` then points at the head's whole list array
   if constexpr (DENSE) {
     n_lists = nqb_all;
   } else if constexpr (BLK == 64) {
@@ -485,19 +492,20 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   } else {
     const int64_t nkb16 = (Lk + 15) >> 4;
     const int32_t* off = p.kq_off + ((int64_t)b * p.H + h) * (nkb16 + 1);
-    const int64_t ka = (int64_t)kb * 4 + 2 * wave;
-    const int32_t lo_a = ka < nkb16 ? off[ka] : 0, hi_a = ka < nkb16 ? off[ka + 1] : 0;
-    const int32_t lo_b = ka + 1 < nkb16 ? off[ka + 1] : 0, hi_b = ka + 1 < nkb16 ? off[ka + 2] : 0;
-    len_a = __builtin_amdgcn_readfirstlane(hi_a - lo_a);
-    len_b = __builtin_amdgcn_readfirstlane(hi_b - lo_b);
-    n_lists = len_a > len_b ? len_a : len_b;  // per wave: the two waves of a tile do not meet (see sync)
-    list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_a;
-    list_b = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride + lo_b;
+    n_lists = 0;  // set per key block below
+    list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride;
+    off16 = off;
   }
+  const int32_t* cur_list = list;  // BLK 16: list and length of the key block being processed
+  int cur_len = 0;
+  // BLK 16, two ways through the tile's four lists.  Workgroups of the first pass (long lists) share every list
+  // between their two waves; in the second pass each wave walks the lists of its own two key blocks, without
+  // barriers or hand-over, which is cheaper where the lists are short.
+  const bool coop = BLK == 16 && long_pass;
   // List entries come 64 at a time (lane l holds entry base + l), so the latency of the list read is paid once per
   // 64 tiles and not in front of every tile's transfers.  The lists are walked front to back.
-  int32_t held_a = -1, held_b = -1;
-  int base_a = -64, base_b = -64;
+  int32_t held_a = -1;
+  int base_a = -64;
   auto entry = [&](const int32_t* lst, int len, int32_t& held, int& base, int i) -> int32_t {
     if (i >= base + 64) {
       base = i & ~63;
@@ -508,7 +516,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   auto block_of = [&](int i) -> int64_t {  // BLK 16: the list position itself
     if constexpr (DENSE) return (int64_t)i;
     else if constexpr (BLK == 64) return (int64_t)entry(list, n_lists, held_a, base_a, i);
-    else return (int64_t)i;
+    else return (int64_t)(coop ? 2 * i + wave : i);  // shared list: the two waves take alternate steps
   };
 
   const float scale = p.scale;
@@ -539,11 +547,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       staged = ((wave == 0 ? lsep : dlp) + start)[r] * (wave == 0 ? kLog2e : scale);
       staged_to = sb + 64 * wave + lane;
     } else {
-      // this wave's half of the tile: 16 queries of entry `qblk` of each of its two lists (an exhausted list: any
+      // this wave's half of the tile: the 16 queries of entries 2t and 2t + 1 of the current list (past its end: any
       // rows, lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
       const int t = (int)qblk;
-      const int32_t ea = t < len_a ? entry(list, len_a, held_a, base_a, t) : -1;
-      const int32_t eb = t < len_b ? entry(list_b, len_b, held_b, base_b, t) : -1;
+      const int32_t ea = 2 * t < cur_len ? entry(cur_list, cur_len, held_a, base_a, 2 * t) : -1;
+      const int32_t eb = 2 * t + 1 < cur_len ? entry(cur_list, cur_len, held_a, base_a, 2 * t + 1) : -1;
       const int64_t sa = ea >= 0 ? (int64_t)ea * 16 : 0, sbk = eb >= 0 ? (int64_t)eb * 16 : 0;
       const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
       const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
@@ -654,28 +662,94 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     if constexpr (BLK == 64) __builtin_amdgcn_s_barrier();
   };
 
-  if (n_lists > 0) {
-    int64_t cur = block_of(0);
-    fetch(cur, H0{});
-    for (int t = 0; t < n_lists; t += 2) {
-      sync();
-      const bool more1 = t + 1 < n_lists;
-      const int64_t nxt1 = more1 ? block_of(t + 1) : cur;
-      if (more1) fetch(nxt1, H1{});
-      compute_tile(cur, H0{});
-      if (!more1) break;
-      sync();
-      const bool more2 = t + 2 < n_lists;
-      cur = more2 ? block_of(t + 2) : nxt1;
-      if (more2) fetch(cur, H0{});
-      compute_tile(nxt1, H1{});
+  auto walk = [&]() {  // all tiles of the current list, double buffered
+    if (n_lists > 0) {
+      int64_t cur = block_of(0);
+      fetch(cur, H0{});
+      for (int t = 0; t < n_lists; t += 2) {
+        sync();
+        const bool more1 = t + 1 < n_lists;
+        const int64_t nxt1 = more1 ? block_of(t + 1) : cur;
+        if (more1) fetch(nxt1, H1{});
+        compute_tile(cur, H0{});
+        if (!more1) break;
+        sync();
+        const bool more2 = t + 2 < n_lists;
+        cur = more2 ? block_of(t + 2) : nxt1;
+        if (more2) fetch(cur, H0{});
+        compute_tile(nxt1, H1{});
+      }
     }
-  }
-
+  };
   E* dkp = (E*)p.dk + (int64_t)b * p.sdkb + (int64_t)h * p.sdkh;
   E* dvp = (E*)p.dv + (int64_t)b * p.sdvb + (int64_t)h * p.sdvh;
-  store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
-  store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
+  if constexpr (BLK == 64) {
+    walk();
+    store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
+    store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
+  } else {
+    // Both waves walk the list of each of the tile's four key blocks together: steps t = wave, wave + 2, ..., entries
+    // 2t and 2t + 1 per step, so a long list is shared by four 16-lane groups and the two waves stay in balance.  At
+    // the end of a list the second wave hands its partial sums over through LDS (the tile buffers are idle then).
+    for (int li = 0; li < (coop ? 4 : 2); li++) {
+      const int64_t kblk = (int64_t)kb * 4 + (coop ? li : 2 * wave + li);
+      if (kblk * 16 >= Lk) break;  // no such key block (shared lists: the same for both waves)
+      key = kblk * 16 + (c & 15);
+      const int32_t lo = __builtin_amdgcn_readfirstlane(off16[kblk]), hi = __builtin_amdgcn_readfirstlane(off16[kblk + 1]);
+      cur_list = list + lo;
+      cur_len = hi - lo;
+      const int steps = (cur_len + 1) >> 1;               // of the list
+      n_lists = coop ? (steps - wave + 1) >> 1 : steps;   // of this wave
+      held_a = -1;
+      base_a = -64;
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's last LDS reads are done before new transfers land
+      load_keys();
+      walk();
+      // lanes c and c + 16 hold partial sums for the same key
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          dkt[dt][r] += __shfl_xor(dkt[dt][r], 16);
+          dvt[dt][r] += __shfl_xor(dvt[dt][r], 16);
+        }
+      const bool live = c < 16 && key < Lk;
+      if (!coop) {
+        store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
+        store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
+        continue;
+      }
+      // wave 1 -> wave 0: 64 values per lane, value i of lane l at float i * 64 + l of the four tile buffers
+      auto slot = [&](int i) -> float* {
+        unsigned char* a = i < 32 ? (i < 16 ? lds_q0 : lds_q1) : (i < 48 ? lds_g0 : lds_g1);
+        return reinterpret_cast<float*>(a) + (i & 15) * 64 + lane;
+      };
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): none of this wave's transfers is still writing the buffers
+      __syncthreads();                      // both waves are done with the tile buffers
+      if (wave == 1) {
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            *slot(dt * 16 + r) = dkt[dt][r];
+            *slot(32 + dt * 16 + r) = dvt[dt][r];
+          }
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            dkt[dt][r] += *slot(dt * 16 + r);
+            dvt[dt][r] += *slot(32 + dt * 16 + r);
+          }
+        store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
+        store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
+      }
+      __syncthreads();  // the hand-over is read before the next list's transfers overwrite it
+    }
+  }
 }
 
 }  // namespace bwd

@@ -119,6 +119,26 @@ def test_selection_backward_with_16_token_blocks_skips_duplicates_and_popular_ke
     assert float(dk[0, :, 16 * (nqb - 3):].abs().max()) == 0.0 and float(dv[0, :, 16 * (nqb - 3):].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("n,kk", [(1040, 2), (2000, 4), (650, 1)])
+def test_selection_backward_with_16_token_blocks_and_very_long_lists(n, kk):
+    """Key blocks that nearly every query block lists: their tiles take the path in which the two waves of a
+    workgroup share each list and hand partial sums over through LDS (lists much longer than 4 * top-k), next to
+    ordinary tiles and a ragged last block."""
+    b, h = 1, 2
+    nqb = -(-n // 16)
+    q, k, v, g = (_randn((b, h, n, 64), 170 + i, torch.bfloat16, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb, 175 + n)
+    idx[0, 0, :, 0] = 9                        # on every list of head 0
+    idx[0, 1, ::2, 0] = nqb - 1                # the ragged last block on every second list of head 1
+    idx[0, 1, 1::2, 0] = 3
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 16, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd, 16)
+    mult = oracle.block_multiplicity(idx, n, 16)
+    wq, wk, wv, _, _ = oracle.attention_grads_formula(q, k, v, g, mult)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+
+
 @pytest.mark.parametrize("b,h,nqb,kk,nkb,hot", [(2, 3, 37, 4, 37, 0), (1, 2, 300, 8, 300, 1), (1, 1, 2600, 4, 650, 2),
                                                 (1, 2, 9000, 2, 40, 3), (1, 1, 1, 1, 1, 0), (1, 2, 70, 64, 70, 0)])
 def test_key_block_lists_match_plain_loops(b, h, nqb, kk, nkb, hot):
