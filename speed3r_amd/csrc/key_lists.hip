@@ -7,7 +7,7 @@
 //
 // Five small kernels, no workspace besides the two outputs:
 //   zero     off[*] = 0
-//   count    histogram of the index entries, block j counted at off[j + 2]
+//   count    histogram of the index entries, block j counted at off[j + 2] (pre-aggregated per workgroup in LDS)
 //   scan     inclusive prefix sum per (b, h): off[j + 1] = first position of block j's list
 //   fill     every entry takes a position with an atomic increment of off[j + 1], which thereby ends up at the END of
 //            block j's list = the start of block j+1's: exactly the offsets array, off[0] = 0 included
@@ -27,27 +27,57 @@ __global__ __launch_bounds__(256) void zero_kernel(int32_t* __restrict__ off, in
   if (i < n) off[i] = 0;
 }
 
-struct Entry {
-  int64_t bh, m;
-  int32_t j;
-};
-__device__ __forceinline__ Entry entry_of(const int32_t* idx, int64_t e, int H, int64_t nqb, int K, int64_t sib, int64_t sih, int64_t sim) {
-  const int kk = (int)(e % K);
-  const int64_t t = e / K;
-  Entry r;
-  r.m = t % nqb;
-  r.bh = t / nqb;
-  const int64_t h = r.bh % H, b = r.bh / H;
-  r.j = idx[b * sib + h * sih + r.m * sim + kk];
-  return r;
-}
+// count and fill share one kernel body.  Neighbouring query blocks name mostly the same key blocks, and atomics on
+// one address serialise in memory, so a workgroup first gathers its 1024 index entries in an LDS hash table (key
+// block -> occurrences), every entry taking its rank among the workgroup's occurrences of its key block with an LDS
+// atomic; one global atomic per DISTINCT key block then adds the count (count pass: at off[j + 2]) or reserves the
+// positions (fill pass: at off[j + 1]), and in the fill pass every entry writes its query block at base + rank.
+// A workgroup stays inside one (b, h): grid.y = B*H, grid.x = chunks of 1024 entries.
+constexpr int kHashSlots = 2048;
 
-__global__ __launch_bounds__(256) void count_kernel(const int32_t* __restrict__ idx, int32_t* __restrict__ off, int H, int64_t nqb, int K,
-                                                     int64_t nkb, int64_t sib, int64_t sih, int64_t sim, int64_t total) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const Entry r = entry_of(idx, e, H, nqb, K, sib, sih, sim);
-  if (r.j >= 0 && (int64_t)r.j + 2 <= nkb) atomicAdd(off + r.bh * (nkb + 1) + r.j + 2, 1);  // the last block's count is not needed
+template <bool FILL>
+__global__ __launch_bounds__(1024) void gather_kernel(const int32_t* __restrict__ idx, int32_t* __restrict__ off, int32_t* __restrict__ list, int H,
+                                                      int64_t nqb, int K, int64_t nkb, int64_t sib, int64_t sih, int64_t sim, int64_t list_stride) {
+  __shared__ int32_t keys[kHashSlots];
+  __shared__ int32_t cnt[kHashSlots];
+  __shared__ int32_t base[kHashSlots];
+  const int t = threadIdx.x;
+  for (int i = t; i < kHashSlots; i += 1024) {
+    keys[i] = -1;
+    cnt[i] = 0;
+  }
+  __syncthreads();
+  const int64_t bh = blockIdx.y;
+  const int64_t hh = bh % H, bb = bh / H;
+  const int64_t e = (int64_t)blockIdx.x * 1024 + t;  // entry within this (b, h)
+  int32_t j = -1, m = 0;
+  if (e < nqb * K) {
+    m = (int32_t)(e / K);
+    j = idx[bb * sib + hh * sih + (int64_t)m * sim + (e - (int64_t)m * K)];
+    if (j < 0 || j >= nkb) j = -1;
+  }
+  int slot = 0, rank = 0;
+  if (j >= 0) {
+    slot = (int)(((uint32_t)j * 2654435761u) >> 21);  // 11 bits
+    while (true) {
+      const int32_t old = atomicCAS(&keys[slot], -1, j);
+      if (old == -1 || old == j) break;
+      slot = (slot + 1) & (kHashSlots - 1);  // at most 1024 keys in 2048 slots: a free slot exists
+    }
+    rank = atomicAdd(&cnt[slot], 1);
+  }
+  __syncthreads();
+  for (int i = t; i < kHashSlots; i += 1024) {
+    const int32_t kj = keys[i];
+    if (kj >= 0) {
+      if (FILL) base[i] = atomicAdd(off + bh * (nkb + 1) + kj + 1, cnt[i]);
+      else if ((int64_t)kj + 2 <= nkb) atomicAdd(off + bh * (nkb + 1) + kj + 2, cnt[i]);  // the last block's count is not needed
+    }
+  }
+  if (FILL) {
+    __syncthreads();
+    if (j >= 0) list[bh * list_stride + base[slot] + rank] = m;
+  }
 }
 
 // one workgroup of 1024 per (b, h): in-place inclusive scan of n values
@@ -71,18 +101,6 @@ __global__ __launch_bounds__(1024) void scan_kernel(int32_t* __restrict__ off, i
   for (int64_t i = lo; i < hi; i++) {
     run += a[i];
     a[i] = run;
-  }
-}
-
-__global__ __launch_bounds__(256) void fill_kernel(const int32_t* __restrict__ idx, int32_t* __restrict__ off, int32_t* __restrict__ list, int H,
-                                                    int64_t nqb, int K, int64_t nkb, int64_t sib, int64_t sih, int64_t sim, int64_t list_stride,
-                                                    int64_t total) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const Entry r = entry_of(idx, e, H, nqb, K, sib, sih, sim);
-  if (r.j >= 0 && r.j < nkb) {
-    const int32_t pos = atomicAdd(off + r.bh * (nkb + 1) + r.j + 1, 1);
-    list[r.bh * list_stride + pos] = (int32_t)r.m;
   }
 }
 
@@ -197,12 +215,13 @@ int launch_key_block_lists(const int32_t* idx, int32_t* kq_list, int32_t* kq_off
   const int64_t bh = (int64_t)B * H;
   const int64_t noff = bh * (nkb + 1), total = bh * nqb * K, nseg = bh * nkb;
   const int64_t g_off = (noff + 255) / 256, g_ent = (total + 255) / 256, g_short = (nseg * 64 + 255) / 256;
-  if (g_off > 0x7fffffffLL || g_ent > 0x7fffffffLL || g_short > 0x7fffffffLL || bh > 0x7fffffffLL)
+  if (g_off > 0x7fffffffLL || g_ent > 0x7fffffffLL || g_short > 0x7fffffffLL || bh > 65535)
     return fail(S3R_ERR_UNSUPPORTED, "s3r_key_block_lists: tensor too large for one launch");
   hipLaunchKernelGGL(kl::zero_kernel, dim3((unsigned)g_off), dim3(256), 0, st, kq_off, noff);
-  hipLaunchKernelGGL(kl::count_kernel, dim3((unsigned)g_ent), dim3(256), 0, st, idx, kq_off, H, nqb, K, nkb, sib, sih, sim, total);
+  const dim3 g_gather((unsigned)((nqb * K + 1023) / 1024), (unsigned)bh);
+  hipLaunchKernelGGL(kl::gather_kernel<false>, g_gather, dim3(1024), 0, st, idx, kq_off, kq_list, H, nqb, K, nkb, sib, sih, sim, list_stride);
   hipLaunchKernelGGL(kl::scan_kernel, dim3((unsigned)bh), dim3(1024), 0, st, kq_off, nkb + 1);
-  hipLaunchKernelGGL(kl::fill_kernel, dim3((unsigned)g_ent), dim3(256), 0, st, idx, kq_off, kq_list, H, nqb, K, nkb, sib, sih, sim, list_stride, total);
+  hipLaunchKernelGGL(kl::gather_kernel<true>, g_gather, dim3(1024), 0, st, idx, kq_off, kq_list, H, nqb, K, nkb, sib, sih, sim, list_stride);
   hipLaunchKernelGGL(kl::sort_short_kernel, dim3((unsigned)g_short), dim3(256), 0, st, kq_list, kq_off, nkb, list_stride, nseg);
   const int64_t g_long = nseg < 4096 ? nseg : 4096;
   hipLaunchKernelGGL(kl::sort_long_kernel, dim3((unsigned)g_long), dim3(256), 0, st, kq_list, kq_off, nkb, list_stride, nseg);
