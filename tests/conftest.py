@@ -28,3 +28,10 @@ def golden():
     import numpy as np
 
     return np.load(ROOT / "tests" / "golden" / "sparse_path_small.npz")
+
+
+@pytest.fixture(scope="session")
+def golden_grads():
+    import numpy as np
+
+    return np.load(ROOT / "tests" / "golden" / "sparse_path_grads_small.npz")

@@ -168,6 +168,19 @@ def test_key_block_lists_match_plain_loops(b, h, nqb, kk, nkb, hot):
             assert flat[o[j]:o[j + 1]] == want[bh][j], (bh, j)
 
 
+@pytest.mark.parametrize("name,block", [("b16", 16), ("b64", 64)])
+def test_selection_forward_and_backward_match_the_brute_force_fixture(golden_grads, name, block):
+    from helpers import from_bf16_bits
+
+    q, k, v, g = (from_bf16_bits(golden_grads[n]).to(DEV) for n in ("q", "k", "v", "dout"))
+    idx = torch.from_numpy(golden_grads[f"{name}_idx"]).to(DEV)
+    o, lse = s3r.select_attn(q, k, v, idx, block, return_lse=True)
+    assert max_abs(o, torch.from_numpy(golden_grads[f"{name}_out"])) <= 2e-2
+    dq, dk, dv = ops.attn_bwd(q, k, v, o, g, lse, idx, block)
+    for got, t in ((dq, "dq"), (dk, "dk"), (dv, "dv")):
+        _close(got, torch.from_numpy(golden_grads[f"{name}_{t}"]), t)
+
+
 def test_operators_are_differentiable_like_the_reference_ones():
     b, h, n = 1, 2, 512
     q, k, v = (_randn((b, h, n, 64), 60 + i, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for i in range(3))

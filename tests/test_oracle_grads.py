@@ -3,6 +3,7 @@ of the library attention and central differences must agree; the key-centric lis
 import math
 
 import numpy as np
+import pytest
 import torch
 import torch.nn.functional as F
 
@@ -97,3 +98,23 @@ def test_key_block_lists_of_the_oracle_hold_every_valid_entry_once_and_in_order(
             assert got[bh][j] == sorted(got[bh][j])
             for m in set(got[bh][j]):
                 assert got[bh][j].count(m) == int((rows[m] == j).sum())
+
+
+@pytest.mark.parametrize("name,block", [("b16", 16), ("b64", 64)])
+def test_gradient_oracle_matches_the_brute_force_fixture(golden_grads, name, block):
+    """The committed vectors come from an fp64 dense softmax under a multiplicity matrix, differentiated by autograd
+    (tests/golden/make_grad_fixtures.py, independent of oracle/): both gradient routes of the oracle must reproduce
+    them, duplicates, skipped and out-of-range entries, an empty row and the ragged last block included."""
+    from helpers import from_bf16_bits
+
+    q, k, v, g = (from_bf16_bits(golden_grads[n]) for n in ("q", "k", "v", "dout"))
+    idx = torch.from_numpy(golden_grads[f"{name}_idx"])
+    want = [torch.from_numpy(golden_grads[f"{name}_{t}"]) for t in ("dq", "dk", "dv")]
+    got = oracle.select_attention_grads_autograd(q, k, v, idx, block, g)
+    for a, w in zip(got, want):
+        assert max_abs(a, w) <= 2e-5 * max(1.0, float(w.abs().max()))
+    mult = oracle.block_multiplicity(idx, q.shape[2], block)
+    dq, dk, dv, o, _ = oracle.attention_grads_formula(q, k, v, g, mult)
+    for a, w in zip((dq, dk, dv), want):
+        assert max_abs(a, w) <= 1e-6 * max(1.0, float(w.abs().max()))
+    assert max_abs(torch.nan_to_num(o.float()), torch.from_numpy(golden_grads[f"{name}_out"])) <= 1e-6
