@@ -434,7 +434,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   // in this lane's store layout.  Issued right after the main loop, so that their latency passes behind the last PV
   // stage instead of in front of the stores.
   const bool merge = p.merge_out != nullptr;
-  float g0[2] = {0.f, 0.f}, g1[2] = {0.f, 0.f};
+  uint32_t g_raw[2] = {0, 0};  // gate pair per query row, bits of the I/O type
   uint4 oc_raw[2][2];  // [dt][gp]
   bool merge_loaded = false;
   auto load_merge_operands = [&]() {
@@ -442,10 +442,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
 #pragma unroll
       for (int qt = 0; qt < 2; qt++) {
         const int64_t row = q0 + qt * 32 + c;
-        if (row < N) {
+        if (row < N) {  // the pair as raw bits: converting it here would wait for the load, and for every transfer before it
           const E* gp = (const E*)p.merge_gate + (int64_t)b * p.sgb + (int64_t)h * p.sgh + row * p.sgn;
-          g0[qt] = (float)gp[0];
-          g1[qt] = (float)gp[1];
+          __builtin_memcpy(&g_raw[qt], gp, 4);
         }
       }
       const E* ocp = (const E*)p.merge_oc + (int64_t)b * p.scb + (int64_t)h * p.sch + (int64_t)qb * p.scm;
@@ -590,6 +589,16 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     }
   }
   if (!merge_loaded) load_merge_operands();
+  float g0[2], g1[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; qt++) {
+    asm volatile("" : "+v"(g_raw[qt]));  // first use of the pair: the wait for its load falls here, behind the last PV stage
+    union { uint16_t u; E e; } lo, hi;
+    lo.u = (uint16_t)g_raw[qt];
+    hi.u = (uint16_t)(g_raw[qt] >> 16);
+    g0[qt] = (float)lo.e;
+    g1[qt] = (float)hi.e;
+  }
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
 #pragma clang fp contract(off)  // the merge rounds each product and the sum separately, like the eager expression
@@ -601,18 +610,20 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
       for (int gp = 0; gp < 2; gp++) {
-        union { E e[8]; uint32_t w[4]; uint4 u; } pc;
-        union { E e[2]; uint32_t w; } t;
-        uint32_t a[2], bw[2];
+        // two values per conversion instruction, words handled as vectors of two (a union of scalars would convert
+        // and mask every value on its own)
+        auto pack2 = [](float x, float y) -> uint32_t {
+          V2 v;
+          v[0] = (E)x;
+          v[1] = (E)y;
+          return __builtin_bit_cast(uint32_t, v);
+        };
+        union { uint32_t w[4]; uint4 u; } pc;
 #pragma unroll
         for (int wi = 0; wi < 2; wi++) {
-          t.e[0] = (E)(ot[dt][qt][8 * gp + 2 * wi] * inv);
-          t.e[1] = (E)(ot[dt][qt][8 * gp + 2 * wi + 1] * inv);
-          a[wi] = t.w;
-          t.e[0] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi] * inv);
-          t.e[1] = (E)(ot[dt][qt][8 * gp + 4 + 2 * wi + 1] * inv);
-          bw[wi] = t.w;
-          const auto r = __builtin_amdgcn_permlane32_swap(a[wi], bw[wi], false, false);
+          const uint32_t a = pack2(ot[dt][qt][8 * gp + 2 * wi] * inv, ot[dt][qt][8 * gp + 2 * wi + 1] * inv);
+          const uint32_t bw = pack2(ot[dt][qt][8 * gp + 4 + 2 * wi] * inv, ot[dt][qt][8 * gp + 4 + 2 * wi + 1] * inv);
+          const auto r = __builtin_amdgcn_permlane32_swap(a, bw, false, false);
           pc.w[wi] = r[0];
           pc.w[2 + wi] = r[1];
         }
@@ -621,13 +632,15 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
           if (!merge) {
             *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
           } else {
-            union { E e[8]; uint4 u; } oc, res;
+            union { uint32_t w[4]; uint4 u; } oc, res;
             oc.u = oc_raw[dt][gp];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-              const float x = round_to<E>(g0[qt] * (float)oc.e[e]);
-              const float y = round_to<E>(g1[qt] * (float)pc.e[e]);
-              res.e[e] = (E)(x + y);
+            for (int wi = 0; wi < 4; wi++) {  // products and sum each rounded to the I/O type, as the eager expression does
+              const V2 o2 = __builtin_bit_cast(V2, oc.w[wi]);
+              const V2 s2 = __builtin_bit_cast(V2, pc.w[wi]);
+              const V2 x2 = __builtin_bit_cast(V2, pack2(g0[qt] * (float)o2[0], g0[qt] * (float)o2[1]));
+              const V2 y2 = __builtin_bit_cast(V2, pack2(g1[qt] * (float)s2[0], g1[qt] * (float)s2[1]));
+              res.w[wi] = pack2((float)x2[0] + (float)y2[0], (float)x2[1] + (float)y2[1]);
             }
             *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = res.u;
           }
