@@ -16,7 +16,9 @@ pi3/models/layers/transformer_head.py (head decoders, linear pixel-shuffle head)
 * heads: three 5-block frame-local decoders on the concatenated outputs of the last local and global blocks, a linear
   pixel-shuffle head for local points and confidence, a small pose head.
 
-All dense GEMMs and the dense attentions are library calls (torch on rocBLAS/hipBLASLt, scaled_dot_product_attention).
+All dense GEMMs are library calls (torch on rocBLAS/hipBLASLt); the frame-local dense attentions run on the package's
+dense flash kernel (the one behind the compressed branch) for bf16/fp16 inference with head_dim 64, else on
+scaled_dot_product_attention.
 Inference only: call under ``torch.no_grad()`` with the module in one dtype (bf16).
 """
 from __future__ import annotations
@@ -49,6 +51,9 @@ class LayerScale(nn.Module):
 
     def forward(self, x: Tensor) -> Tensor:
         return x * self.gamma
+
+    def add_to(self, residual: Tensor, x: Tensor) -> Tensor:  # residual + gamma * x in one pass
+        return torch.addcmul(residual, x, self.gamma)
 
 
 class DenseAttentionRope(nn.Module):
@@ -84,6 +89,11 @@ class DenseAttentionRope(nn.Module):
         q, k, v = self.qkv(x).view(b, n, 3, h, c // h).permute(2, 0, 3, 1, 4).unbind(0)
         pos = xpos if self.rope is not None else None
         q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
+        if x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and c // h == 64 and not torch.is_grad_enabled():
+            # the package's dense flash kernel (the compressed branch's attention), written straight into [B,N,H,D]
+            o = torch.empty((b, n, h, c // h), dtype=x.dtype, device=x.device)
+            ops.compressed_attn_topk(q, k, v, None, out=o.permute(0, 2, 1, 3))
+            return self.proj(o.view(b, n, c))
         o = F.scaled_dot_product_attention(q, k, v)
         return self.proj(o.transpose(1, 2).reshape(b, n, c))
 
@@ -100,8 +110,10 @@ class Block(nn.Module):
         self.ls2 = LayerScale(dim, init_values) if init_values else nn.Identity()
 
     def forward(self, x: Tensor, xpos: Optional[Tensor] = None) -> Tensor:
-        x = x + self.ls1(self.attn(self.norm1(x), xpos=xpos))
-        return x + self.ls2(self.mlp(self.norm2(x)))
+        a = self.attn(self.norm1(x), xpos=xpos)
+        x = self.ls1.add_to(x, a) if isinstance(self.ls1, LayerScale) else x + a
+        m = self.mlp(self.norm2(x))
+        return self.ls2.add_to(x, m) if isinstance(self.ls2, LayerScale) else x + m
 
 
 class PatchEncoder(nn.Module):
@@ -127,10 +139,12 @@ class PatchEncoder(nn.Module):
         return torch.cat((cls, patch.permute(0, 2, 3, 1).reshape(1, gh * gw, -1)), dim=1)
 
     def forward(self, imgs: Tensor) -> Tensor:  # [F,3,H,W] -> patch tokens [F, gh*gw, dim]
-        f = imgs.shape[0]
-        x = self.patch_embed(imgs)
-        gh, gw = x.shape[-2:]
-        x = x.flatten(2).transpose(1, 2)
+        f, ch, hh, ww = imgs.shape
+        p = self.patch
+        gh, gw = hh // p, ww // p
+        # kernel == stride: the convolution is one GEMM over the unfolded patches (same parameters as the Conv2d)
+        x = imgs[:, :, :gh * p, :gw * p].reshape(f, ch, gh, p, gw, p).permute(0, 2, 4, 1, 3, 5).reshape(f, gh * gw, ch * p * p)
+        x = F.linear(x, self.patch_embed.weight.reshape(self.patch_embed.out_channels, -1), self.patch_embed.bias)
         x = torch.cat((self.cls_token.expand(f, -1, -1), x), dim=1) + self._pos(gh, gw)
         x = torch.cat((x[:, :1], self.register_tokens.expand(f, -1, -1), x[:, 1:]), dim=1)
         for blk in self.blocks:

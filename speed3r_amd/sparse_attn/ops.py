@@ -81,7 +81,8 @@ def pool_qkv_packed(qkv: torch.Tensor, num_heads: int, block: int) -> Tuple[torc
 
 def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], topk: Optional[int],
                          softmax_scale: Optional[float] = None, return_scores: bool = False,
-                         return_lse: bool = False, materialize_scores: Optional[bool] = None):
+                         return_lse: bool = False, materialize_scores: Optional[bool] = None,
+                         out: Optional[torch.Tensor] = None):
     """Dense attention over pooled tokens plus, if ``topk`` is given, the top-k columns of the
     raw scores per query row.
 
@@ -94,6 +95,9 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Ten
     ``v=None`` asks for the indices alone (``o`` is returned as ``None``; fused selection only): the
     attention output and the indices come from two different kernels, and a caller with two streams runs
     them side by side, see :func:`sparse_global_attention`.
+
+    ``out``: a ``[B,H,Lq,D]`` tensor (or view, any strides on the first three dimensions, e.g. the
+    ``permute(0, 2, 1, 3)`` of a ``[B,Lq,H,D]`` buffer) that receives the attention output instead of a fresh one.
     """
     indices_only = v is None
     if indices_only:
@@ -109,7 +113,10 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Ten
     lk = k.shape[2]
     assert k.shape == (b, h, lk, d) and v.shape == (b, h, lk, d), "k/v shape mismatch"
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    o = None if indices_only else torch.empty_like(q, memory_format=torch.contiguous_format)
+    if out is not None:
+        assert not indices_only and out.shape == q.shape and out.dtype == q.dtype and out.device == q.device \
+            and out.stride(-1) == 1, "out must be a [B,H,Lq,D] tensor of q's dtype and device, last dimension contiguous"
+    o = None if indices_only else out if out is not None else torch.empty_like(q, memory_format=torch.contiguous_format)
     idx = torch.empty((b, h, lq, topk), dtype=torch.int32, device=q.device) if topk else None
     fused_ok = (q.dtype != torch.float32 and d == 64 and topk in (1, 2, 4, 8, 16, 32) and lk <= (1 << 21)
                 and _lib.lib_has_fused_topk())

@@ -102,3 +102,17 @@ def test_layer_module_refuses_cpu_tensors():
     m = SparseFlashAttentionRope(dim=128, num_heads=2, block_size=8, topk=2)
     with torch.no_grad(), pytest.raises(Exception):
         m(torch.zeros((1, 128, 128)))
+
+
+def test_patch_embedding_as_one_gemm_equals_the_convolution():
+    """The model's patch embedding (unfold + linear on the Conv2d's parameters) against F.conv2d, fp32 on the CPU."""
+    import torch.nn.functional as F
+    from speed3r_amd.model.pi3_sparse_like import PatchEncoder
+    torch.manual_seed(0)
+    enc = PatchEncoder(dim=32, depth=0, num_heads=2, patch=14, grid=(3, 2), num_register=4)
+    imgs = torch.rand(2, 3, 45, 31)                       # not multiples of 14: the convolution drops the remainder
+    want = F.conv2d(imgs, enc.patch_embed.weight, enc.patch_embed.bias, stride=14).flatten(2).transpose(1, 2)
+    got = enc(imgs)                                       # depth 0: tokens = norm(embedding + position) without cls/registers
+    f, gh, gw = 2, 3, 2
+    x = torch.cat((enc.cls_token.expand(f, -1, -1), want), dim=1) + enc._pos(gh, gw)
+    assert torch.allclose(got, enc.norm(x)[:, 1:], atol=1e-5)
