@@ -155,6 +155,16 @@ int s3r_norm_rope(const void* x, void* y, const int32_t* pos, const void* cos_ta
                   int dtype, void* stream);
 
 /*
+ * LayerNorm over the channels of token rows:  y[r,:] = (x[r,:] - mean_r) * rstd_r * w + b, fp32 statistics, one
+ * rounding to the I/O dtype.  Replaces, for inference, the nn.LayerNorm modules in front of the attention layers and
+ * the MLPs (norm1 / norm2, pi3/models/layers/block.py:281,296,312,315).
+ *   x, y: [rows, C] in the I/O dtype with row strides sx, sy (elements; multiples of 16 bytes); w, b: [C] (b may be
+ *   NULL).  C: a multiple of 16 bytes worth of elements, at most 4096 (two-byte types) or 2048 (fp32).
+ */
+int s3r_layer_norm(const void* x, void* y, const void* w, const void* b, float eps, int64_t rows, int C,
+                   int64_t sx, int64_t sy, int dtype, void* stream);
+
+/*
  * Gated merge of the two branches, written in the [B,N,H*D] layout the output projection
  * reads:  out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d].
  * Replaces the einops/broadcast expression in pi3/models/layers/sparse_attention.py:127-136.

@@ -34,6 +34,7 @@ SIGNATURES = {
                                       *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
     "s3r_norm_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
                               c_int, c_int, c_int64, c_int, *_i64x3, c_int64, c_int64, c_int, c_void_p]),
+    "s3r_layer_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int64, c_int64, c_int, c_void_p]),
     "s3r_gated_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int,
                                 *_i64x3, *_i64x3, *_i64x3, c_int, c_void_p]),
     "s3r_attn_bwd_delta": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, *_i64x3, *_i64x3,

@@ -1,0 +1,108 @@
+// LayerNorm over the channel dimension of token rows ([rows, C], C up to 4096 two-byte or 2048 four-byte values), HBM bound.
+//
+// Replaces the pre-attention / pre-MLP norms around the attention layers (norm1 / norm2 of
+// pi3/models/layers/block.py:281,296,312,315; nn.LayerNorm, eps 1e-6) for inference: y = (x - mean) * rstd * w + b
+// with fp32 statistics and one rounding to the I/O dtype, as torch's kernel computes it.
+//
+// One wavefront owns a row: lane l holds the 16-byte chunks l, l + 64, ... of the row in registers (NCH chunks, two
+// for 1024 bf16 channels), so the row is read once; sum and centred sum of squares are xor-shuffle folds over the 64
+// lanes.  Four rows per workgroup, no LDS, no barrier.
+#include "s3r_common.h"
+
+namespace s3r {
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const T* __restrict__ x, T* __restrict__ y, const T* __restrict__ w,
+                                                         const T* __restrict__ b, float eps, int64_t rows, int C,
+                                                         int64_t sx, int64_t sy) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;  // whole waves leave: the shuffles below stay wave-uniform
+  const int nchunks = C / VEC;
+  const T* xr = x + row * sx;
+  float v[NCH][VEC];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    const int ch = lane + 64 * i;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (ch < nchunks) raw = *reinterpret_cast<const uint4*>(xr + ch * VEC);
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+      v[i][j] = to_f32(e[j]);
+      s += v[i][j];
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) s += __shfl_xor(s, off);
+  const float mean = s / (float)C;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; i++)
+    if (lane + 64 * i < nchunks) {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) q += (v[i][j] - mean) * (v[i][j] - mean);
+    }
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) q += __shfl_xor(q, off);
+  const float rstd = 1.0f / sqrtf(q / (float)C + eps);
+  T* yr = y + row * sy;
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    const int ch = lane + 64 * i;
+    if (ch < nchunks) {
+      uint4 wr = *reinterpret_cast<const uint4*>(w + ch * VEC);
+      uint4 br = make_uint4(0, 0, 0, 0);
+      if (b != nullptr) br = *reinterpret_cast<const uint4*>(b + ch * VEC);
+      const T* we = reinterpret_cast<const T*>(&wr);
+      const T* be = reinterpret_cast<const T*>(&br);
+      uint4 out;
+      T* oe = reinterpret_cast<T*>(&out);
+#pragma unroll
+      for (int j = 0; j < VEC; j++) oe[j] = from_f32<T>((v[i][j] - mean) * rstd * to_f32(we[j]) + to_f32(be[j]));
+      *reinterpret_cast<uint4*>(yr + ch * VEC) = out;
+    }
+  }
+}
+
+template <typename T>
+static void launch_layer_norm(const void* x, void* y, const void* w, const void* b, float eps, int64_t rows, int C,
+                              int64_t sx, int64_t sy, hipStream_t st) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int per_lane = (C / VEC + 63) / 64;  // 16-byte chunks per lane
+  dim3 grid((unsigned)((rows + 3) / 4)), blk(256);
+#define S3R_LN(NCH)                                                                                                   \
+  hipLaunchKernelGGL((layer_norm_kernel<T, NCH>), grid, blk, 0, st, (const T*)x, (T*)y, (const T*)w, (const T*)b, eps, \
+                     rows, C, sx, sy)
+  if (per_lane <= 1) S3R_LN(1);
+  else if (per_lane <= 2) S3R_LN(2);
+  else if (per_lane <= 4) S3R_LN(4);
+  else S3R_LN(8);
+#undef S3R_LN
+}
+
+}  // namespace s3r
+
+using namespace s3r;
+
+extern "C" int s3r_layer_norm(const void* x, void* y, const void* w, const void* b, float eps, int64_t rows, int C,
+                              int64_t sx, int64_t sy, int dtype, void* stream) {
+  if (!x || !y || !w) return fail(S3R_ERR_BAD_ARG, "s3r_layer_norm: null pointer");
+  if (rows <= 0 || C <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_layer_norm: non-positive size");
+  if (dtype != S3R_F32 && dtype != S3R_BF16 && dtype != S3R_F16) return fail(S3R_ERR_UNSUPPORTED, "s3r_layer_norm: dtype %d", dtype);
+  const int es = elt_size(dtype);
+  const int vec = 16 / es;
+  if (C % vec != 0 || C / vec > 8 * 64)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_layer_norm: %d channels (built for multiples of %d up to %d)", C, vec, 8 * 64 * vec);
+  if (sx < C || sy < C) return fail(S3R_ERR_BAD_ARG, "s3r_layer_norm: row stride below the row length");
+  if (!aligned16(x) || !aligned16(y) || !aligned16(w) || (b && !aligned16(b)) || (sx * es) % 16 || (sy * es) % 16)
+    return fail(S3R_ERR_BAD_ARG, "s3r_layer_norm: pointers and row strides must be multiples of 16 bytes");
+  if ((rows + 3) / 4 > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_layer_norm: too many rows for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == S3R_F32) launch_layer_norm<float>(x, y, w, b, eps, rows, C, sx, sy, st);
+  else if (dtype == S3R_BF16) launch_layer_norm<bf16_t>(x, y, w, b, eps, rows, C, sx, sy, st);
+  else launch_layer_norm<f16_t>(x, y, w, b, eps, rows, C, sx, sy, st);
+  return check_launch("s3r_layer_norm");
+}

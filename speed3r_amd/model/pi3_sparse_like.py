@@ -56,6 +56,15 @@ class LayerScale(nn.Module):
         return torch.addcmul(residual, x, self.gamma)
 
 
+def token_norm(norm: nn.LayerNorm, x: Tensor) -> Tensor:
+    """The block norms: the package's one-pass kernel for inference on the GPU, the torch module otherwise."""
+    if x.is_cuda and not torch.is_grad_enabled() and norm.elementwise_affine and x.dtype == norm.weight.dtype:
+        y = ops.layer_norm(x, norm.weight, norm.bias, norm.eps)
+        if y is not None:
+            return y
+    return norm(x)
+
+
 class DenseAttentionRope(nn.Module):
     """Dense attention inside each sequence of the batch (one frame), optional qk-norm and RoPE2D."""
 
@@ -110,9 +119,9 @@ class Block(nn.Module):
         self.ls2 = LayerScale(dim, init_values) if init_values else nn.Identity()
 
     def forward(self, x: Tensor, xpos: Optional[Tensor] = None) -> Tensor:
-        a = self.attn(self.norm1(x), xpos=xpos)
+        a = self.attn(token_norm(self.norm1, x), xpos=xpos)
         x = self.ls1.add_to(x, a) if isinstance(self.ls1, LayerScale) else x + a
-        m = self.mlp(self.norm2(x))
+        m = self.mlp(token_norm(self.norm2, x))
         return self.ls2.add_to(x, m) if isinstance(self.ls2, LayerScale) else x + m
 
 
@@ -149,7 +158,7 @@ class PatchEncoder(nn.Module):
         x = torch.cat((x[:, :1], self.register_tokens.expand(f, -1, -1), x[:, 1:]), dim=1)
         for blk in self.blocks:
             x = blk(x)
-        return self.norm(x)[:, 1 + self.register_tokens.shape[1]:]
+        return token_norm(self.norm, x)[:, 1 + self.register_tokens.shape[1]:]
 
 
 class HeadDecoder(nn.Module):

@@ -253,6 +253,30 @@ def norm_rope(x: torch.Tensor, positions: Optional[torch.Tensor], cos_tab: Optio
     return y
 
 
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> Optional[torch.Tensor]:
+    """``F.layer_norm(x, (C,), weight, bias, eps)`` over the last dimension of token rows in one pass (inference).
+
+    Returns None when the library has no kernel for the shape (rows that are not a multiple of 16 bytes or longer
+    than 512 16-byte chunks, a tensor whose leading dimensions do not collapse to one row stride)."""
+    _need_device(x)
+    _forward_only(x)
+    c = x.shape[-1]
+    vec = 16 // x.element_size()
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or c % vec or c // vec > 512 or x.numel() == 0:
+        return None
+    x2 = x.reshape(-1, c) if x.is_contiguous() else None
+    if x2 is None:
+        return None
+    w = weight.detach().to(x.dtype).contiguous()
+    b = bias.detach().to(x.dtype).contiguous() if bias is not None else None
+    y = torch.empty_like(x2)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().s3r_layer_norm(x2.data_ptr(), y.data_ptr(), w.data_ptr(), b.data_ptr() if b is not None else None,
+                                       float(eps), x2.shape[0], c, x2.stride(0), y.stride(0), _code(x), _stream(x))
+    _lib.check(rc, "s3r_layer_norm")
+    return y.view(x.shape)
+
+
 def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, o_cmp: torch.Tensor,
                       gate: torch.Tensor, block: int, softmax_scale: Optional[float] = None) -> Optional[torch.Tensor]:
     """``select_attn`` with ``gated_merge`` in its epilogue -> ``[B,N,H*D]``; bit-identical to the two calls, without the

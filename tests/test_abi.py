@@ -70,6 +70,9 @@ def test_backward_entry_points_validate_on_the_host():
     assert bwd(q_st=(64 * 64, 64 * 64, 1 << 20)) == _lib.S3R_ERR_UNSUPPORTED  # row stride beyond the 32-bit tile offsets
     assert bwd(q_st=(64 * 64, 64 * 64, 60)) == _lib.S3R_ERR_BAD_ARG          # rows not 16-byte aligned
     assert b"s3r_attn_bwd" in L.s3r_last_error()
+    assert L.s3r_layer_norm(None, one, one, None, 1e-6, 1, 64, 64, 64, _lib.S3R_BF16, None) == _lib.S3R_ERR_BAD_ARG
+    assert L.s3r_layer_norm(one, one, one, None, 1e-6, 1, 12, 64, 64, _lib.S3R_BF16, None) == _lib.S3R_ERR_UNSUPPORTED
+    assert b"s3r_layer_norm" in L.s3r_last_error()
     assert L.s3r_key_block_lists(None, one, one, 1, 1, 4, 4, 4, *z3, 16, None) == _lib.S3R_ERR_BAD_ARG
     assert L.s3r_key_block_lists(one, one, one, 1, 1, 4, 4, 4, *z3, 15, None) == _lib.S3R_ERR_BAD_ARG      # list_stride < nqb * K
     assert L.s3r_key_block_lists(one, one, one, 1, 1, 1 << 30, 4, 4, *z3, 1 << 32, None) == _lib.S3R_ERR_UNSUPPORTED

@@ -327,3 +327,33 @@ def test_forward_only_guard():
     x = torch.zeros((1, 1, 64, 64), dtype=torch.bfloat16, device=DEV, requires_grad=True)
     with pytest.raises(RuntimeError, match="forward-only"):
         s3r.pool_mean(x, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,c", [(1, 8), (7, 1024), (1030, 1024), (5, 136), (3, 2048), (9, 512)])
+def test_layer_norm_matches_fp64_closed_form(dtype, rows, c):
+    """s3r_layer_norm against (x - mean) / sqrt(var + eps) * w + b evaluated in fp64 on the same inputs; the result is
+    rounded once to the I/O dtype: half an ulp of the output plus the fp32 error of the statistics."""
+    from speed3r_amd.sparse_attn import ops
+    g = torch.Generator().manual_seed(rows * 131 + c)
+    x = (torch.randn(rows, c, generator=g) * 3 + 0.5).to(dtype).to("cuda:0")
+    w = (torch.randn(c, generator=g)).to(dtype).to("cuda:0")
+    b = (torch.randn(c, generator=g)).to(dtype).to("cuda:0")
+    for bias in (b, None):
+        got = ops.layer_norm(x, w, bias, 1e-6)
+        assert got is not None and got.shape == x.shape and got.dtype == dtype
+        xd = x.double()
+        mean = xd.mean(-1, keepdim=True)
+        var = ((xd - mean) ** 2).mean(-1, keepdim=True)
+        ref = (xd - mean) / torch.sqrt(var + 1e-6) * w.double() + (bias.double() if bias is not None else 0.0)
+        ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[dtype]
+        assert ((got.double() - ref).abs() <= ulp * ref.abs() + 1e-5).all()
+    # constant rows: zero variance, the output is the bias
+    xc = torch.full((4, c), 2.5, dtype=dtype, device="cuda:0")
+    assert torch.equal(ops.layer_norm(xc, w, b, 1e-6), b.expand(4, c))
+
+
+def test_layer_norm_declines_rows_it_has_no_kernel_for():
+    from speed3r_amd.sparse_attn import ops
+    w = torch.ones(12, dtype=torch.bfloat16, device="cuda:0")
+    assert ops.layer_norm(torch.ones(3, 12, dtype=torch.bfloat16, device="cuda:0"), w, None, 1e-6) is None
