@@ -101,6 +101,9 @@ int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int
  *   o:   I/O dtype [B,H,N,D];  lse: optional fp32 [B,H,N] contiguous.
  * Keys beyond N in a partial last block are masked out; a query block with no valid entry
  * gives zeros.  block in {4,16,32,64}, D <= 64 (MFMA paths: block 64 or 16, D == 64, bf16/fp16, K <= 64).
+ * The reference's larger blocks (128, 256; topk_blocksparse_attention.py:862) are the caller's to rewrite, as the
+ * Python operator does: the list of a query block serves each of its 64-row parts, a listed key block j becomes the
+ * entries r*j .. r*j+r-1 (r = block/64), and the call is made with block 64 and K*r entries per row.
  */
 int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* idx,
                     void* o, float* lse,

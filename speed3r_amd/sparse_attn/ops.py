@@ -163,6 +163,20 @@ def topk_rows(scores: torch.Tensor, k: int) -> torch.Tensor:
     return idx
 
 
+def _as_64_token_blocks(idx: torch.Tensor, block: int, n: int) -> torch.Tensor:
+    """Index lists over blocks of 128 or 256 tokens rewritten for the 64-token kernels.
+
+    A query block of ``r * 64`` rows is ``r`` consecutive 64-row blocks with the same list, and a listed key block is
+    the run of its ``r`` 64-token blocks in order, so the rewritten tensor is ``[B,H,ceil(N/64),K*r]``: the same keys
+    in the same order for every query row (entries below zero stay -1; runs reaching beyond ``N`` are cut by the
+    kernels' own ``start >= N`` rule)."""
+    r = block // 64
+    b, h, nqb, kk = idx.shape
+    sub = torch.arange(r, device=idx.device, dtype=torch.int32)
+    fine = torch.where(idx[..., None] >= 0, idx[..., None] * r + sub, idx.new_full((), -1))
+    return fine.reshape(b, h, nqb, kk * r).repeat_interleave(r, dim=2)[:, :, :-(-n // 64)].contiguous()
+
+
 def select_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor, block: int,
                 softmax_scale: Optional[float] = None, return_lse: bool = False):
     """Attention of each ``block``-row query block over the key blocks listed in ``idx``."""
@@ -175,6 +189,8 @@ def select_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Te
     assert k.shape == q.shape and v.shape == q.shape, "q, k, v must share a shape"
     nqb = -(-n // block)
     assert idx.shape[:3] == (b, h, nqb), f"topk_idx shape {tuple(idx.shape)} does not match {(b, h, nqb, 'K')}"
+    if block in (128, 256):
+        idx, block = _as_64_token_blocks(idx, block, n), 64
     kk = idx.shape[3]
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
     o = torch.empty_like(q, memory_format=torch.contiguous_format)
@@ -293,6 +309,9 @@ def select_attn_merge(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: to
     assert idx.shape[:3] == (b, h, nqb), f"topk_idx shape {tuple(idx.shape)} does not match {(b, h, nqb, 'K')}"
     assert o_cmp.shape == (b, h, nqb, d), f"o_cmp shape {tuple(o_cmp.shape)} != {(b, h, nqb, d)}"
     assert gate.shape == (b, h, n, 2), f"gate shape {tuple(gate.shape)} != {(b, h, n, 2)}"
+    if block in (128, 256):  # 64-row query blocks share their parent's list and its row of the compressed output
+        o_cmp = o_cmp.repeat_interleave(block // 64, dim=2)[:, :, :-(-n // 64)].contiguous()
+        idx, block = _as_64_token_blocks(idx, block, n), 64
     if q.dtype == torch.float32 or d != 64 or block not in (64, 16) or idx.shape[3] > 64:
         return None
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
@@ -447,6 +466,9 @@ def select_attn_autograd(q, k, v, idx, block, softmax_scale=None):
     """:func:`select_attn`, differentiable in q, k, v where the backward kernels are built."""
     if not _wants_grad(q, k, v):
         return select_attn(q, k, v, idx, block, softmax_scale)
+    if block in (128, 256):
+        assert idx.shape[2] == -(-q.shape[2] // block), "topk_idx does not match the number of query blocks"
+        idx, block = _as_64_token_blocks(idx, block, q.shape[2]), 64
     if not bwd_supported(q, block):
         raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64, blocks of 64 or 16 tokens")
     return _SelectAttnFn.apply(q, k, v, idx, block, softmax_scale)

@@ -19,15 +19,14 @@ def topk_blocksparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
     """Every ``block_size``-row query block attends to the key blocks its ``topk_idx`` row lists.
 
     ``-1`` (or any index whose block starts at or beyond ``seq_len``) means "skip".  Returns the
-    attention output with q's shape and dtype.  The reference accepts bf16/fp16 only; fp32 is
+    attention output with q's shape and dtype.  Blocks of 128 and 256 tokens run on the 64-token kernels: the same
+    list serves the 2 (4) 64-row parts of a query block and a listed key block is visited as its 2 (4) 64-token parts.  The reference accepts bf16/fp16 only; fp32 is
     accepted here as well.  ``softmax_scale`` defaults to ``1/sqrt(head_dim)``.
     """
     assert q.dtype in (torch.bfloat16, torch.float16, torch.float32)
     assert q.dtype == k.dtype and k.dtype == v.dtype
     assert topk_idx.dtype == torch.int32
     assert block_size in {4, 16, 32, 64, 128, 256}
-    if block_size > 64:
-        raise NotImplementedError("topk_blocksparse_attention: block_size above 64 is not built")
     batch, nheads, seq_len, _ = q.shape
     assert topk_idx.shape[0] == batch
     assert topk_idx.shape[1] == nheads

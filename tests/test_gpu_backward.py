@@ -260,3 +260,18 @@ def test_backward_at_full_size_on_sampled_blocks():
                 want_dk, want_dv = ds.T @ qf, p.T @ gf
             assert max_abs(dk[0, h, keys], want_dk) <= 2e-2 * max(1.0, float(want_dk.abs().max()))
             assert max_abs(dv[0, h, keys], want_dv) <= 2e-2 * max(1.0, float(want_dv.abs().max()))
+
+
+@pytest.mark.parametrize("n,block,kk", [(1041, 128, 3), (1500, 256, 2)])
+def test_selection_backward_with_blocks_of_128_and_256_tokens(n, block, kk):
+    """The differentiable operator at the reference's larger block sizes (run as runs of 64-token blocks) against
+    autograd through the oracle at the large block size itself."""
+    b, h, dtype = 1, 2, torch.bfloat16
+    nqb = -(-n // block)
+    q, k, v, g = (_randn((b, h, n, 64), 60 + i, dtype, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb, 70 + n)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o = s3r.topk_blocksparse_attention(qd, kd, vd, idx.to(DEV), block)
+    o.backward(g.to(DEV))
+    wq, wk, wv = oracle.select_attention_grads_autograd(q, k, v, idx, block, g)
+    _close(qd.grad, wq, "dq"); _close(kd.grad, wk, "dk"); _close(vd.grad, wv, "dv")

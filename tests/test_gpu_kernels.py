@@ -357,3 +357,38 @@ def test_layer_norm_declines_rows_it_has_no_kernel_for():
     from speed3r_amd.sparse_attn import ops
     w = torch.ones(12, dtype=torch.bfloat16, device="cuda:0")
     assert ops.layer_norm(torch.ones(3, 12, dtype=torch.bfloat16, device="cuda:0"), w, None, 1e-6) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("n,block,k,with_invalid", [(512, 128, 2, False), (1041, 128, 4, True), (1041, 256, 3, True),
+                                                    (2000, 256, 8, False), (100, 128, 1, False), (300, 256, 2, True)])
+def test_select_blocks_of_128_and_256_tokens_match_oracle(dtype, n, block, k, with_invalid):
+    """The reference operator also takes blocks of 128 and 256 tokens (topk_blocksparse_attention.py:862); here they run
+    as runs of 64-token blocks.  Against the oracle at the large block size itself: ragged lengths, skipped and
+    duplicated entries, an empty query block; the fused merge against merge(oracle selection)."""
+    h = 2
+    nqb = -(-n // block)
+    q = _randn((1, h, n, 64), n, dtype, 0.5)
+    kk = _randn((1, h, n, 64), n + 1, dtype, 0.5)
+    v = _randn((1, h, n, 64), n + 2, dtype)
+    g = torch.Generator().manual_seed(n + k)
+    lo, hi = (-1, nqb + 1) if with_invalid else (0, nqb)
+    idx = torch.randint(lo, hi, (1, h, nqb, k), generator=g, dtype=torch.int32)
+    if with_invalid:
+        idx[0, 0, 0, :] = -1
+        if k > 1:
+            idx[0, 1, nqb - 1, 1] = idx[0, 1, nqb - 1, 0]
+    o = s3r.topk_blocksparse_attention(q.to(DEV), kk.to(DEV), v.to(DEV), idx.to(DEV), block)
+    o_ref = oracle.select_attention(q, kk, v, idx, block, out_dtype=torch.float32)
+    assert o.dtype == dtype and o.shape == q.shape
+    assert max_abs(o, o_ref) <= TOL[dtype]
+    if with_invalid:
+        assert float(o[0, 0, :min(block, n)].float().abs().max()) == 0.0
+    pooled_rows = _randn((1, h, nqb, 64), n + 3, dtype)
+    gate = torch.sigmoid(_randn((1, h, n, 2), n + 4, torch.float32)).to(dtype)
+    two = s3r.gated_merge(pooled_rows.to(DEV), o, gate.to(DEV), block)
+    fused = s3r.select_attn_merge(q.to(DEV), kk.to(DEV), v.to(DEV), idx.to(DEV), pooled_rows.to(DEV), gate.to(DEV), block)
+    if dtype == torch.float32:
+        assert fused is None                     # the fused epilogue is a 16-bit kernel
+    else:
+        assert torch.equal(fused, two)

@@ -32,7 +32,7 @@ def _oracle_out(m, x, xpos, idx):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 4e-2), (torch.float32, 2e-4)])
-@pytest.mark.parametrize("n,block_size,topk", [(320, 8, 2), (200, 8, 4), (160, 4, 4), (64, 8, 1)])
+@pytest.mark.parametrize("n,block_size,topk", [(320, 8, 2), (200, 8, 4), (160, 4, 4), (64, 8, 1), (1100, 16, 2)])
 def test_layer_matches_the_oracle(dtype, tol, n, block_size, topk):
     b, dim, heads = 2, 128, 2
     m = _make(dim, heads, block_size, topk, dtype, seed=n)
