@@ -17,6 +17,8 @@
 // block with no valid entry gives zeros; up to 64 entries per query block.
 #include "select_common.h"
 #include "attn_params.h"
+#include <stdlib.h>
+#include <string.h>
 
 namespace s3r {
 namespace b16 {
@@ -27,7 +29,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 typedef std::integral_constant<int, 0> H0;
 typedef std::integral_constant<int, 1> H1;
 
-template <typename E>
+// UNION: the wave walks the union of its four lists, see below (default); otherwise pairs of list entries.
+template <typename E, bool UNION>
 __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nqb, int ngrp, int nwg_per_bh, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
@@ -216,24 +219,232 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
       for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[jj].v, ot[dt][QT]);
   };
 
-  const int nsteps = p.K;
-  if (nsteps > 0) {
-    fetch(0, H0{});
-    for (int i = 0; i < nsteps; i++) {
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 1 (previous step) are done
-      fetch(i, H1{});
-      __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 0) has landed
-      compute(i, H0{});
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 0 are done
-      if (i + 1 < nsteps) {
-        fetch(i + 1, H0{});
-        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 1) has landed
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  if constexpr (UNION) {
+    // Neighbouring query blocks list mostly the same key blocks.  The wave therefore walks the UNION of its four
+    // lists: a tile is two distinct key blocks A, B (rows 0-15, 16-31), fetched once, and every one of the 64 queries
+    // whose block lists A (B) uses its 16 scores against A (B); cnt bytes say how often query block j lists the
+    // block (0: not at all, its scores are masked; above 1: a duplicated entry, the probabilities count that often).
+    // The visiting order differs from the lists' order, which changes fp32 summation order only.
+    uint64_t rem[4];
+    bool exact = false;  // second walk: running maximum
+    auto pop = [&](int32_t& blk, uint32_t& cnts) {  // next distinct key block and its four multiplicities, or -1
+      blk = -1;
+      cnts = 0;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (blk < 0 && rem[j] != 0) blk = __builtin_amdgcn_readlane(my_idx[j], __ffsll((unsigned long long)rem[j]) - 1);
+      if (blk >= 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const uint64_t hit = __ballot(my_idx[j] == blk) & rem[j];
+          rem[j] &= ~hit;
+          cnts |= (uint32_t)__popcll(hit) << (8 * j);
+        }
       }
-      compute(i, H1{});
+    };
+    auto fetch_u = [&](int buf, int32_t ba, int32_t bb) {  // K and V rows of blocks A, B -> buffers buf (no B: block 0 again)
+      char* kb = buf ? k_buf[1] : k_buf[0];
+      char* vb = buf ? v_buf[1] : v_buf[0];
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const int32_t blk = s == 0 ? ba : bb;
+        const int64_t start = (int64_t)(blk < 0 ? 0 : blk) * 16;
+        const int last = (int)((N - start < 16 ? N - start : 16) - 1);
+        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + start * p.svn), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int ldsrow = 16 * s + 8 * t + lr;
+          int row = 8 * t + lr;
+          row = row < last ? row : last;
+          const uint32_t kc = (uint32_t)(((lane & 7) ^ (ldsrow & 7)) * 16);
+          const uint32_t vc = (uint32_t)(((lane & 7) ^ (((ldsrow >> 1) & 1) << 2)) * 16);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(kb + (2 * s + t) * 1024), 16,
+                                                   (uint32_t)row * krow + kc, 0, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(vb + (2 * s + t) * 1024), 16,
+                                                   (uint32_t)row * vrow + vc, 0, 0, 0);
+        }
+      }
+    };
+    auto compute_u = [&](int buf, int32_t ba, uint32_t ca, int32_t bb, uint32_t cb) {
+      const char* kb = buf ? k_buf[1] : k_buf[0];
+      const char* vb = buf ? v_buf[1] : v_buf[0];
+      V8 ak[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(kb + (kr_off ^ (ks << 5)));
+        ak[ks] = as_v8<E>(f);
+      }
+      V8 vfr[2][2];
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) {
+          const char* a0 = vb + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+          Frag f;
+          f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+          f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+          vfr[jj][dt] = as_v8<E>(f);
+        }
+      const int nka = (int)(N - (int64_t)ba * 16 < 16 ? N - (int64_t)ba * 16 : 16);
+      const int nkb = bb < 0 ? 0 : (int)(N - (int64_t)bb * 16 < 16 ? N - (int64_t)bb * 16 : 16);
+      const int mine = c >> 4;
+      // The three stages of a 32-query half (one half after the other: interleaving the two halves' stages was slower).
+      f32x16 st[2];
+      union { V8 v; } pf[2][2];
+      auto scores = [&](auto qt_tag) {
+        constexpr int QT = decltype(qt_tag)::value;
+#pragma unroll
+        for (int r = 0; r < 16; r++) st[QT][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) st[QT] = Mma<E>::mma(ak[ks], bq[QT][ks], st[QT]);
+      };
+      auto softmax = [&](auto qt_tag) {
+        constexpr int QT = decltype(qt_tag)::value;
+        const uint32_t pa = (ca >> (16 * QT)) & 0xffffu, pb = (cb >> (16 * QT)) & 0xffffu;  // the half's two query blocks
+        const int wa = (int)(mine ? pa >> 8 : pa & 0xffu), wb = (int)(mine ? pb >> 8 : pb & 0xffu);
+        // register r: key row 4hh + 8((r%8)/4) + r%4 of block A (r < 8) or B (r >= 8).  A block that the lane's query
+        // block does not list is left out through two per-lane constants (its maximum is dropped and its exponent gets
+        // -inf added); only the ragged last block needs per-register masks.
+        if (__any((wa && nka < 16) || (wb && nkb < 16))) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            const int row = 4 * hh + 8 * (j >> 2) + (j & 3);
+            if (row >= nka) st[QT][j] = -INFINITY;
+            if (row >= nkb) st[QT][8 + j] = -INFINITY;
+          }
+        }
+        // Softmax reference.  First walk (exact == false): a query's reference is the maximum over the first tile that
+        // holds a block of its list and then stays (softmax is shift invariant), so later tiles need no maximum, no
+        // comparison and no pass over the accumulators; probabilities may exceed 1, and a row sum that ends up huge or
+        // not finite sends the group through a second walk with the running maximum (exact == true).
+        const bool unset = m_i[QT] == -INFINITY && (wa | wb) != 0;
+        if (exact || __any(unset)) {
+          float mxa = st[QT][0], mxb = st[QT][8];
+#pragma unroll
+          for (int r = 1; r < 8; r++) {
+            mxa = fmaxf(mxa, st[QT][r]);
+            mxb = fmaxf(mxb, st[QT][8 + r]);
+          }
+          float mx = fmaxf(wa ? mxa : -INFINITY, wb ? mxb : -INFINITY);
+          mx = xh_max(mx) * sl2;
+          const float m_new = (exact || unset) ? fmaxf(m_i[QT], mx) : m_i[QT];
+          if (__any(m_new != m_i[QT])) {
+            const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - (m_new == -INFINITY ? 0.f : m_new));  // 0 while m_i is -inf
+            l_i[QT] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
+          }
+          m_i[QT] = m_new;
+        }
+        const float m_use = m_i[QT] == -INFINITY ? 0.f : m_i[QT];
+        const float nega = wa ? -m_use : -INFINITY, negb = wb ? -m_use : -INFINITY;  // -inf: every probability 0
+        const bool dup = __any(wa > 1 || wb > 1);
+        const float fa = (float)wa, fb = (float)wb;
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) {
+            float x0 = __builtin_amdgcn_exp2f(fmaf(st[QT][8 * jj + e], sl2, jj == 0 ? nega : negb));
+            float x1 = __builtin_amdgcn_exp2f(fmaf(st[QT][8 * jj + e + 1], sl2, jj == 0 ? nega : negb));
+            if (dup) {  // a list that names the block more than once attends it that often
+              x0 *= jj == 0 ? fa : fb;
+              x1 *= jj == 0 ? fa : fb;
+            }
+            V2 pk;
+            pk[0] = (E)x0;
+            pk[1] = (E)x1;
+            pf[QT][jj].v[e] = pk[0];
+            pf[QT][jj].v[e + 1] = pk[1];
+            l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
+          }
+      };
+      auto values = [&](auto qt_tag) {
+        constexpr int QT = decltype(qt_tag)::value;
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+          for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[QT][jj].v, ot[dt][QT]);
+      };
+      // (wave-uniform) does some query of the half list A or B?
+      const bool act0 = ((ca | cb) & 0xffffu) != 0, act1 = ((ca | cb) >> 16) != 0;
+      if (act0) {
+        scores(H0{});
+        softmax(H0{});
+        values(H0{});
+      }
+      if (act1) {
+        scores(H1{});
+        softmax(H1{});
+        values(H1{});
+      }
+    };
+    for (int pass = 0; pass < 2; pass++) {
+      exact = pass == 1;
+#pragma unroll
+      for (int j = 0; j < 4; j++) rem[j] = __ballot(my_idx[j] >= 0);
+      int32_t a0, b0;
+      uint32_t ca0, cb0;
+      pop(a0, ca0);
+      pop(b0, cb0);
+      if (a0 >= 0) {
+        int buf = 0;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): (second walk) the first walk's last reads are done
+        fetch_u(0, a0, b0);
+        while (true) {
+          int32_t a1, b1;
+          uint32_t ca1, cb1;
+          pop(a1, ca1);
+          pop(b1, cb1);
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the previous tile's reads of the other buffers are done
+          if (a1 >= 0) {
+            fetch_u(buf ^ 1, a1, b1);
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the current tile has landed
+          } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+          }
+          compute_u(buf, a0, ca0, b0, cb0);
+          if (a1 < 0) break;
+          a0 = a1; ca0 = ca1; b0 = b1; cb0 = cb1;
+          buf ^= 1;
+        }
+      }
+      const float big = 1.2676506e30f;  // 2^100
+      if (exact || !__any(!(l_i[0] < big) || !(l_i[1] < big))) break;
+      // rare: some reference was far too low; start over with the running maximum
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) ot[dt][qt][r] = 0.f;
+      m_i[0] = m_i[1] = -INFINITY;
+      l_i[0] = l_i[1] = 0.f;
     }
-  }
+  } else {
+  const int nsteps = p.K;
+    if (nsteps > 0) {
+      fetch(0, H0{});
+      for (int i = 0; i < nsteps; i++) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 1 (previous step) are done
+        fetch(i, H1{});
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 0) has landed
+        compute(i, H0{});
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffers 0 are done
+        if (i + 1 < nsteps) {
+          fetch(i + 1, H0{});
+          __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): unit (i, 1) has landed
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        }
+        compute(i, H1{});
+      }
+    }
+  
+}
 
   // output: as in the 64-token kernels (one exchange with lane ^ 32 per packed word, 16-byte stores).  With merge
   // operands the gated merge runs here (gate pair of the row, the compressed output of the row's 16-token block; the
@@ -303,10 +514,18 @@ int launch_select_b16(const AttnParams& p, int dtype, void* stream) {
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)total), blk(256);
-  if (dtype == S3R_BF16)
-    hipLaunchKernelGGL((b16::select_b16_kernel<bf16_t>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total);
-  else
-    hipLaunchKernelGGL((b16::select_b16_kernel<f16_t>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total);
+  // default: the union walk; S3R_B16_KERNEL=pairs picks the walk over pairs of list entries (kept as a cross-check)
+  static const bool pairs = [] {
+    const char* e = getenv("S3R_B16_KERNEL");
+    return e != nullptr && strcmp(e, "pairs") == 0;
+  }();
+#define S3R_B16(E, U) hipLaunchKernelGGL((b16::select_b16_kernel<E, U>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total)
+  if (dtype == S3R_BF16) {
+    if (pairs) S3R_B16(bf16_t, false); else S3R_B16(bf16_t, true);
+  } else {
+    if (pairs) S3R_B16(f16_t, false); else S3R_B16(f16_t, true);
+  }
+#undef S3R_B16
   return check_launch("select_b16_kernel");
 }
 

@@ -392,3 +392,24 @@ def test_select_blocks_of_128_and_256_tokens_match_oracle(dtype, n, block, k, wi
         assert fused is None                     # the fused epilogue is a 16-bit kernel
     else:
         assert torch.equal(fused, two)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_select_block16_handles_scores_far_above_the_reference(dtype):
+    """The 16-token kernel fixes a query's softmax reference at the first tile that holds one of its blocks; blocks
+    visited later with logits ~140 (base 2) above it overflow the row sums and must send the group through the walk
+    with a running maximum.  Also the mild case (probabilities above 1 without overflow: fp16 overflows earlier)."""
+    for gain in (12.0, 2.0):
+        g = torch.Generator().manual_seed(5)
+        n, h = 256, 2
+        q = torch.randn((1, h, n, 64), generator=g).to(dtype)
+        k = (torch.randn((1, h, n, 64), generator=g) * 0.01).to(dtype)
+        k[:, :, 128:192] = (q[:, :, 0:64] * gain).to(dtype)     # key blocks 8..11 line up with the queries of blocks 0..3
+        v = torch.randn((1, h, n, 64), generator=g).to(dtype)
+        nqb = n // 16
+        idx = torch.stack([torch.tensor([(m + 1) % nqb, 8 + (m % 4), (m + 5) % nqb, 9], dtype=torch.int32) for m in range(nqb)])
+        idx = idx.view(1, 1, nqb, 4).expand(1, h, nqb, 4).contiguous()
+        o = s3r.select_attn(q.to(DEV), k.to(DEV), v.to(DEV), idx.to(DEV), 16)
+        ref = oracle.select_attention(q, k, v, idx, 16, out_dtype=torch.float32)
+        assert torch.isfinite(o.float()).all()
+        assert max_abs(o, ref) <= 2e-2
