@@ -216,8 +216,9 @@ def test_select_matches_oracle(dtype, n, block, k):
 @pytest.mark.parametrize("n,k,with_invalid", [(96, 4, False), (1041, 32, False), (1041, 32, True), (200, 7, True), (16, 1, False),
                                               (2000, 64, True), (70, 3, True)])
 def test_select_block16_matches_oracle(dtype, n, k, with_invalid):
-    """16-token blocks (the reference layer's own setting) run on the MFMA kernel that pairs query blocks: ragged
-    lengths, group tails (query-block counts that are not multiples of four), skipped and duplicated entries."""
+    """16-token blocks (the reference layer's own setting) on their MFMA kernel (a wave walks the union of four query
+    blocks' lists): ragged lengths, group tails (query-block counts that are not multiples of four), skipped and
+    duplicated entries."""
     h, block = 2, 16
     nqb = -(-n // block)
     q = _randn((1, h, n, 64), n, dtype, 0.5)
@@ -413,3 +414,30 @@ def test_select_block16_handles_scores_far_above_the_reference(dtype):
         ref = oracle.select_attention(q, k, v, idx, 16, out_dtype=torch.float32)
         assert torch.isfinite(o.float()).all()
         assert max_abs(o, ref) <= 2e-2
+
+
+def test_select_block16_pair_walk_matches_oracle():
+    """The cross-check walk of the 16-token kernel (S3R_B16_KERNEL=pairs, read once per process, hence the subprocess)
+    against the oracle and against the default union walk: ragged length, skipped and duplicated entries."""
+    import subprocess, sys, textwrap
+    code = textwrap.dedent("""
+        import os, sys, torch
+        sys.path.insert(0, ".")
+        sys.path.insert(0, "tests")
+        import oracle, speed3r_amd as s3r
+        n, h, k = 1041, 2, 32
+        nqb = -(-n // 16)
+        g = torch.Generator().manual_seed(11)
+        q, kk, v = ((torch.randn((1, h, n, 64), generator=g) * s).to(torch.bfloat16) for s in (0.5, 0.5, 1.0))
+        idx = torch.randint(-1, nqb + 1, (1, h, nqb, k), generator=g, dtype=torch.int32)
+        idx[0, 0, 0, :] = -1
+        idx[0, 1, 5, 1] = idx[0, 1, 5, 0]
+        o = s3r.select_attn(q.cuda(), kk.cuda(), v.cuda(), idx.cuda(), 16)
+        ref = oracle.select_attention(q, kk, v, idx, 16, out_dtype=torch.float32)
+        err = (o.float().cpu() - ref).abs().max().item()
+        assert err <= 2e-2, err
+        print("ok", err)
+    """)
+    env = dict(__import__("os").environ, S3R_B16_KERNEL="pairs")
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110, env=env)
+    assert res.returncode == 0, res.stdout + res.stderr
