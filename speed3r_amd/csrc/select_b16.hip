@@ -2,7 +2,7 @@
 // the reference layer's own setting, block_size**2 = 16 with 32 blocks per query block
 // (pi3/models/layers/sparse_attention.py:73,98,125; kernel topk_blocksparse_attention.py:35-128).
 //
-// One wavefront owns four consecutive query blocks (64 queries) of one head; four independent waves per workgroup.
+// One wavefront owns four consecutive query blocks (64 queries) of one head; one wave per workgroup.
 // The 32x32x16 MFMA wants 32 keys and 32 queries per tile, a query block has only 16 of each per list entry, so a
 // tile pairs TWO query blocks with ONE list entry of each: rows 0-15 of the key half tile hold the block the first
 // query block lists at position i, rows 16-31 the block the second one lists at position i.  S^T = K Q^T then has
@@ -25,19 +25,26 @@ namespace b16 {
 using namespace sel;
 
 constexpr int kHalfBytes = 32 * 128;
+#ifndef S3R_B16_WAVES
+#define S3R_B16_WAVES 1
+#endif
+// wavefronts (groups of four query blocks) per workgroup; the waves do not interact.  One: the unions differ in size
+// (cfg-3-like lists: 32 to 127 distinct blocks), and a workgroup keeps its slots until its slowest wave is done
+// (4 waves: 1.71 ms, 2: 1.50 ms, 1: 1.42 ms at 266 496 tokens, top-32).
+constexpr int kWaves = S3R_B16_WAVES;
 constexpr float kLog2e = 1.4426950408889634f;
 typedef std::integral_constant<int, 0> H0;
 typedef std::integral_constant<int, 1> H1;
 
 // UNION: the wave walks the union of its four lists, see below (default); otherwise pairs of list entries.
 template <typename E, bool UNION>
-__global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nqb, int ngrp, int nwg_per_bh, int total_wg) {
+__global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p, int nqb, int ngrp, int nwg_per_bh, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[4 * kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[4 * kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[4 * kHalfBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[4 * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[kWaves * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[kWaves * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kWaves * kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kWaves * kHalfBytes];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
   const int wg = vid - bh * nwg_per_bh;
   const int b = bh / p.H;
   const int h = bh - b * p.H;
-  const int grp = wg * 4 + wave;  // group of four query blocks = 64 queries
+  const int grp = wg * kWaves + wave;  // group of four query blocks = 64 queries
   if (grp >= ngrp) return;
 
   const int64_t N = p.Lq;
@@ -509,11 +516,11 @@ __global__ __launch_bounds__(256, 2) void select_b16_kernel(AttnParams p, int nq
 int launch_select_b16(const AttnParams& p, int dtype, void* stream) {
   const int64_t nqb = (p.Lq + 15) / 16;
   const int64_t ngrp = (nqb + 3) / 4;
-  const int64_t nwg = (ngrp + 3) / 4;
+  const int64_t nwg = (ngrp + b16::kWaves - 1) / b16::kWaves;
   const int64_t total = nwg * p.B * p.H;
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)total), blk(256);
+  dim3 grid((unsigned)total), blk(64 * b16::kWaves);
   // default: the union walk; S3R_B16_KERNEL=pairs picks the walk over pairs of list entries (kept as a cross-check)
   static const bool pairs = [] {
     const char* e = getenv("S3R_B16_KERNEL");
