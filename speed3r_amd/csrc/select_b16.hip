@@ -273,17 +273,17 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
         }
       }
     };
-    auto compute_u = [&](int buf, int32_t ba, uint32_t ca, int32_t bb, uint32_t cb) {
+    V8 ak[4];       // K fragments of the current tile
+    V8 vfr[2][2];   // V^T fragments of the current tile [jj][dt]
+    auto load_frags = [&](int buf) {
       const char* kb = buf ? k_buf[1] : k_buf[0];
       const char* vb = buf ? v_buf[1] : v_buf[0];
-      V8 ak[4];
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
         Frag f;
         f.u = *reinterpret_cast<const uint4*>(kb + (kr_off ^ (ks << 5)));
         ak[ks] = as_v8<E>(f);
       }
-      V8 vfr[2][2];
 #pragma unroll
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
@@ -294,6 +294,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
           f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
           vfr[jj][dt] = as_v8<E>(f);
         }
+    };
+    auto compute_u = [&](int32_t ba, uint32_t ca, int32_t bb, uint32_t cb) {  // on the fragments in registers
       const int nka = (int)(N - (int64_t)ba * 16 < 16 ? N - (int64_t)ba * 16 : 16);
       const int nkb = bb < 0 ? 0 : (int)(N - (int64_t)bb * 16 < 16 ? N - (int64_t)bb * 16 : 16);
       const int mine = c >> 4;
@@ -400,22 +402,28 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       if (a0 >= 0) {
         int buf = 0;
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): (second walk) the first walk's last reads are done
+        // Two tiles in flight: a tile's fragments go to registers in one go, which frees its buffers for the tile
+        // after the next before any arithmetic starts.
         fetch_u(0, a0, b0);
+        int32_t a1, b1;
+        uint32_t ca1, cb1;
+        pop(a1, ca1);
+        pop(b1, cb1);
+        if (a1 >= 0) fetch_u(1, a1, b1);
         while (true) {
-          int32_t a1, b1;
-          uint32_t ca1, cb1;
-          pop(a1, ca1);
-          pop(b1, cb1);
-          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the previous tile's reads of the other buffers are done
-          if (a1 >= 0) {
-            fetch_u(buf ^ 1, a1, b1);
-            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the current tile has landed
-          } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-          }
-          compute_u(buf, a0, ca0, b0, cb0);
+          if (a1 >= 0) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the current tile has landed (the next one may be in flight)
+          else __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+          load_frags(buf);
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments are in registers, the buffers are free
+          int32_t a2, b2;
+          uint32_t ca2, cb2;
+          pop(a2, ca2);
+          pop(b2, cb2);
+          if (a2 >= 0) fetch_u(buf, a2, b2);
+          compute_u(a0, ca0, b0, cb0);
           if (a1 < 0) break;
           a0 = a1; ca0 = ca1; b0 = b1; cb0 = cb1;
+          a1 = a2; ca1 = ca2; b1 = b2; cb1 = cb2;
           buf ^= 1;
         }
       }
