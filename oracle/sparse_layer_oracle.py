@@ -15,9 +15,14 @@ The two operators, pooling and merge inside ``sparse_layer`` are the functions o
 Pins (tests/test_oracle_layer.py): rope2d against the textbook rotation (for head_dim 4 every half is one plane
 rotated by ``pos`` radians), against its invariants (position 0 is the identity, norms are preserved, the y half
 ignores x, inner products depend on position differences only) and, in fp64, against a complex-number
-formulation written independently; block_positions against hand-computed cases.  ``sparse_layer`` composes pinned
-parts in the order of the cited lines; nothing in the reference holds an output of the layer, so the composition
-itself is checked only by reading (parity unpinned at that level).
+formulation written independently; block_positions against hand-computed cases.  ``sparse_layer``
+(tests/test_oracle_layer_composition.py): with every key block selected the layer must equal
+``proj(g0 * broadcast(compressed row) + g1 * dense attention)`` built from explicit per-head row ranges of the weight
+matrices, ``F.layer_norm``, ``F.scaled_dot_product_attention``, a complex-number rotation and plain block means; with
+fewer blocks, the block-masked dense softmax under ``torch.topk`` of the pooled scores; gate extremes isolate each
+branch (the (0, 1) extreme is the reference's eager dense layer, sparse_attention.py:39-58).  Each check also asserts
+that ten plausible mistakes (swapped split order, swapped gate pairing, norm before pooling, rounded or first-token
+block positions, exchanged y/x, ...) land far outside the tolerance.
 """
 from __future__ import annotations
 
