@@ -8,7 +8,9 @@
  * (head_dim) stride of every q/k/v/o tensor is 1.  Launches are asynchronous on `stream`
  * (a hipStream_t passed as void*; NULL = the default stream).  Every function returns
  * S3R_OK or a negative error code and never throws; s3r_last_error() gives the message of
- * the calling thread's last failure.  Nothing is allocated, no global state is kept.
+ * the calling thread's last failure.  No entry point allocates memory.  State kept between calls: the S3R_*
+ * environment switches (read once, on first use) and the built-in score buffer of
+ * s3r_compressed_attn_topk_static; nothing else.
  */
 #ifndef SPEED3R_HIP_H
 #define SPEED3R_HIP_H
@@ -79,6 +81,27 @@ int s3r_compressed_attn_topk(const void* q, const void* k, const void* v,
                              int64_t svb, int64_t svh, int64_t svn,
                              int64_t sob, int64_t soh, int64_t som,
                              float softmax_scale, int dtype, void* stream);
+
+/*
+ * s3r_compressed_attn_topk with its score buffer built into the library: allocates nothing.
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It is the `scores != NULL` path of
+ * s3r_compressed_attn_topk (any I/O dtype, any K a power of two <= 64; indices selected from exactly the stored
+ * fp32 scores, so results equal that call bit for bit) with the B*H*Lq*Lk scores held in a file-scope device array
+ * of S3R_STATIC_SCORES_MAX floats (96 MiB per GPU the library runs on, kept until the process ends).  Larger
+ * problems return S3R_ERR_UNSUPPORTED.  `o` and `topk_idx` are both required.  The first call on a device looks up
+ * that device's copy of the array (no allocation; make it outside a graph capture).  All calls on one GPU share
+ * the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ */
+#define S3R_STATIC_SCORES_MAX (24u * 1024u * 1024u)
+int s3r_compressed_attn_topk_static(const void* q, const void* k, const void* v,
+                                    void* o, float* lse, int32_t* topk_idx,
+                                    int B, int H, int Lq, int Lk, int D, int K,
+                                    int64_t sqb, int64_t sqh, int64_t sqm,
+                                    int64_t skb, int64_t skh, int64_t skn,
+                                    int64_t svb, int64_t svh, int64_t svn,
+                                    int64_t sob, int64_t soh, int64_t som,
+                                    float softmax_scale, int dtype, void* stream);
 
 /*
  * Row-wise exact top-k of a materialised fp32 score matrix (same ordering rule as above).

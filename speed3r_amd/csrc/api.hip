@@ -4,6 +4,7 @@
 #include "attn_bwd.h"
 #include <stdlib.h>
 #include <string.h>
+#include <mutex>
 
 namespace s3r {
 
@@ -61,6 +62,57 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
   if (rc != S3R_OK) return rc;
   if (topk_idx != nullptr) rc = s3r_topk_rows(scores, topk_idx, (int64_t)B * H * Lq, Lk, Lk, K, stream);
   return rc;
+}
+
+// ---- the entry point that allocates nothing --------------------------------------------------
+// Score buffer of s3r_compressed_attn_topk_static: device memory owned by the code object, one copy per GPU at
+// its own address, held until the process ends.  The name below is only a handle for hipGetSymbolAddress; host
+// code uses the looked-up address.
+static __device__ __align__(256) float scratch[S3R_STATIC_SCORES_MAX];
+
+namespace s3r {
+
+static constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices] = {};   // per device, filled on the first call there
+static std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`; looked up once per device.
+static int static_scores(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(S3R_ERR_HIP, "s3r_compressed_attn_topk_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(S3R_ERR_HIP, "s3r_compressed_attn_topk_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return S3R_OK;
+}
+
+}  // namespace s3r
+
+extern "C" int s3r_compressed_attn_topk_static(const void* q, const void* k, const void* v, void* o, float* lse, int32_t* topk_idx,
+                                               int B, int H, int Lq, int Lk, int D, int K,
+                                               int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
+                                               int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t som,
+                                               float softmax_scale, int dtype, void* stream) {
+  if (!o || !topk_idx) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk_static: null pointer");
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk_static: non-positive size");
+  const unsigned long long need = (unsigned long long)B * H * Lq * (unsigned long long)Lk;
+  if (need > S3R_STATIC_SCORES_MAX)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk_static: B*H*Lq*Lk = %llu scores exceed the built-in buffer of %u "
+                                     "(use s3r_compressed_attn_topk)", need, (unsigned)S3R_STATIC_SCORES_MAX);
+  float* scores = nullptr;
+  int rc = static_scores(&scores);
+  if (rc != S3R_OK) return rc;
+  // every score of the B*H*Lq*Lk the selection reads is written by the attention kernel first: nothing to clear
+  return s3r_compressed_attn_topk(q, k, v, o, lse, topk_idx, scores, B, H, Lq, Lk, D, K, sqb, sqh, sqm, skb, skh, skn,
+                                  svb, svh, svn, sob, soh, som, softmax_scale, dtype, stream);
 }
 
 namespace s3r {
