@@ -30,8 +30,10 @@ PEAK_HBM_GBS = 8000.0
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # The chip's clock governor needs some tens of back-to-back launches to settle under this load (the first
+    # launches after an idle period run up to 40 % slower), so the default warm-up is long; a step is 1.8 ms.
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
                     help="cfg1-cfg4: one sparse global-attention layer call; cfg5: end-to-end Pi3_Sparse-style forward (frames/s)")
     ap.add_argument("--frames", type=int, default=100, help="cfg5: number of 518x392 frames")
@@ -51,12 +53,26 @@ def parse_args():
     return ap.parse_args()
 
 
+def _cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(q, k, v, gate, block, topk, heads):
-    """Times the oracle (eager fp32 PyTorch + numpy top-k) on `heads` heads of the workload."""
+    """Times the oracle (eager fp32 PyTorch + numpy top-k) on `heads` heads of the workload, on as many threads as
+    this process may use (its CPU affinity, not the machine's core count: the box's share can be smaller)."""
     import torch
 
     import oracle
 
+    usable = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = max(1, min(usable, int(os.environ.get("OMP_NUM_THREADS", usable))))
+    torch.set_num_threads(threads)
     hs = slice(0, heads)
     qs, ks, vs, gs = (t[:, hs].float() for t in (q, k, v, gate))
     t0 = time.perf_counter()
@@ -67,6 +83,8 @@ def cpu_baseline(q, k, v, gate, block, topk, heads):
         "value": dt * 1e3 * total_heads / heads,
         "unit": "ms",
         "cores": torch.get_num_threads(),
+        "host_cpus": os.cpu_count(),
+        "cpu_model": _cpu_model(),
         "kind": "port",
         "sample": f"oracle (eager fp32 PyTorch + numpy top-k) on heads 0..{heads - 1} of {total_heads}, all tokens: "
                   f"{dt:.2f} s measured, scaled x{total_heads // heads} to the full layer",
@@ -132,7 +150,7 @@ def run_end_to_end(args) -> int:
 
 def run_backward(args, cfg, qd, kd, vd, block, topk) -> int:
     """Backward of the selection operator and of the compressed (dense) operator on the forward's tensors: HIP events
-    around delta, the key-centric lists (torch device sort), the dQ kernel and the dK/dV kernel."""
+    around delta, the key-centric lists (`s3r_key_block_lists`), the dQ kernel and the dK/dV kernel."""
     import torch
 
     import speed3r_amd as s3r
@@ -315,9 +333,10 @@ def main() -> int:
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
-            # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a plain copy (profiles/); measured for the
-            # default workload only
+            # HBM bytes per launch: not measured inside this run; the figure is the one rocprofv3 FETCH_SIZE / WRITE_SIZE
+            # gave for this kernel on this workload, scaled by a plain copy (file named in traffic_source)
             "traffic": 2.34e9 if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
+            "traffic_source": "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md" if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
         },
     }
     if not args.no_cpu_baseline:

@@ -55,6 +55,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const int hh = lane >> 5;
   const int c = lane & 31;
 
+  // everything the index row's address and the Q transfers need, fetched from the argument block in ONE round trip
+  // (the compiler would otherwise fetch each argument where it is first used: three dependent trips before the row)
+  if constexpr (!DENSE)
+    asm volatile("" ::"s"(p.H), "s"(nqg), "s"(nqb), "s"(total_wg), "s"(p.idx), "s"(p.sib), "s"(p.sih), "s"(p.sim), "s"(p.K), "s"(p.q),
+                 "s"(p.sqb), "s"(p.sqh), "s"(p.sqm), "s"(p.Lq));
   const int w = blockIdx.x;
   const int xcd = w & 7, slot = w >> 3;
   const int per = total_wg >> 3, rem = total_wg & 7;
@@ -78,6 +83,14 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const E* vp = (const E*)p.v + (int64_t)b * p.svb + (int64_t)h * p.svh;
   E* op = (E*)p.o + (int64_t)b * p.sob + (int64_t)h * p.soh;
   const int32_t* idx_row = DENSE ? nullptr : p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim;
+  // The index row is the head of the longest dependency chain of the start-up (row -> first K tile -> first scores):
+  // its load is the wave's first memory instruction, ahead of the Q transfers in the vector memory queue, one entry
+  // per lane; the scheduling barrier keeps the compiler from sinking it to its first use.
+  int32_t my_idx = -1;
+  if constexpr (!DENSE) {
+    if (lane < p.K) my_idx = __builtin_nontemporal_load(idx_row + lane);
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   auto k_half = [&](auto hf) -> E* {
     if constexpr (decltype(hf)::value == 0) return reinterpret_cast<E*>(lds_k0) + wave * kHalf;
@@ -113,7 +126,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   }
 
   // index list: full tiles go through the pipeline, occurrences of the ragged last block come after it
-  int32_t my_idx = -1;
   const int32_t ragged_blk = (N & 63) ? (int32_t)(N >> 6) : -1;
   bool my_valid = false;
   uint64_t todo = 0;
@@ -132,27 +144,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     dense_next = dense_begin;
     dense_end = dense_begin + n_full;
   } else {
-    // The list comes through the scalar cache (s_load): a vector load would wait in the vector memory queue behind
-    // the Q transfers and behind the other waves' tile transfers, and the first K transfer waits for the list.
-    const int32_t __attribute__((address_space(4)))* srow = (const int32_t __attribute__((address_space(4)))*)idx_row;
-    if (p.K == 16) {
-      int32_t sidx[16];
-#pragma unroll
-      for (int i = 0; i < 16; i++) sidx[i] = srow[i];
-#pragma unroll
-      for (int i = 0; i < 16; i++) my_idx = lane == i ? sidx[i] : my_idx;
-    } else if (p.K == 32) {
-      int32_t sidx[32];
-#pragma unroll
-      for (int i = 0; i < 32; i++) sidx[i] = srow[i];
-#pragma unroll
-      for (int i = 0; i < 32; i++) my_idx = lane == i ? sidx[i] : my_idx;
-    } else {
-      for (int i = 0; i < p.K; i++) {  // other lengths: one entry at a time
-        const int32_t v = srow[i];
-        my_idx = lane == i ? v : my_idx;
-      }
-    }
     my_valid = my_idx >= 0 && (int64_t)my_idx * 64 < N;
     todo = __ballot(my_valid && my_idx != ragged_blk);
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
@@ -343,8 +334,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         pk[1] = (E)x1;
         pf[qt][KT][jj][e8] = pk[0];
         pf[qt][KT][jj][e8 + 1] = pk[1];
-        l_i[qt] += x0;  // row sums over the unrounded probabilities, as the reference's tl.sum(p) before p.to(v.dtype)
-        l_i[qt] += x1;
+        // row sums over the unrounded probabilities, as the reference's tl.sum(p) before p.to(v.dtype); the pair is
+        // added first: two additions chained on the sum stall the second one behind the exponential's result
+        l_i[qt] += x0 + x1;
         asm volatile("" : "+v"(pf[qt][KT][jj]), "+v"(l_i[qt]));
       }
       __builtin_amdgcn_sched_barrier(0);
