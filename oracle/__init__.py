@@ -19,6 +19,7 @@ from .sparse_attention_oracle import (  # noqa: F401
     sparse_global_attention,
 )
 from .sparse_layer_oracle import rope2d, block_positions, sparse_layer  # noqa: F401,E402
+from .model_oracle import pi3_sparse_like_forward  # noqa: F401,E402
 from .attention_grad_oracle import (  # noqa: F401,E402
     select_attention_grads_autograd,
     compressed_attention_grads_autograd,

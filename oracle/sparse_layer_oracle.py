@@ -64,9 +64,9 @@ def block_positions(xpos: torch.Tensor, block: int) -> torch.Tensor:
 
 def sparse_layer(x, w_qkv, b_qkv, w_gate, b_gate, w_proj, b_proj, num_heads: int, block: int, topk: int,
                  xpos: Optional[torch.Tensor] = None, qn_w=None, qn_b=None, kn_w=None, kn_b=None,
-                 rope_base: float = 100.0, idx_override: Optional[torch.Tensor] = None):
+                 rope_base: float = 100.0, idx_override: Optional[torch.Tensor] = None, ln_eps: float = 1e-5):
     """One forward of the layer on CPU tensors of one dtype.  ``qn_*``/``kn_*``: LayerNorm(head_dim) affine
-    parameters (None: no qk-norm).  Returns dict(out, idx, o_cmp, o_sel)."""
+    parameters (None: no qk-norm), ``ln_eps`` their epsilon.  Returns dict(out, idx, o_cmp, o_sel)."""
     b, n, c = x.shape
     h, d = num_heads, c // num_heads
     dt = x.dtype
@@ -76,7 +76,7 @@ def sparse_layer(x, w_qkv, b_qkv, w_gate, b_gate, w_proj, b_proj, num_heads: int
     def norm(t, w, bias):
         if w is None:
             return t
-        return F.layer_norm(t.float(), (d,), w.float(), bias.float()).to(dt)
+        return F.layer_norm(t.float(), (d,), w.float(), bias.float(), ln_eps).to(dt)
 
     q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)
     qc, kc, vc = (ops.pool_mean(t, block, out_dtype=dt) for t in (q, k, v))

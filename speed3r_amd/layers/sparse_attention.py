@@ -27,6 +27,28 @@ from ..sparse_attn.flash_attention_topk import flash_attn_topk_func
 from .pos_embed import RoPE2D, block_positions
 
 
+def norm_rope_fused_or_eager(t: Tensor, norm: nn.Module, rope, pos: Optional[Tensor]) -> Tensor:
+    """qk-norm, cast and RoPE of one ``[B,H,N,D]`` tensor (reference sparse_attention.py:103-110,120-124): one fused
+    kernel where it is built -- a tensor on the GPU, head_dim 64, ``nn.Identity`` or an affine ``nn.LayerNorm`` of
+    exactly that type, the package's RoPE2D or no rotation -- and the separate torch modules otherwise (any other norm
+    module, a LayerNorm without affine parameters, another rope).  Same rounding points either way, except that the
+    kernel takes the LayerNorm parameters in the tokens' dtype (fp32 parameters under autocast are rounded to it)."""
+    fused_norm = isinstance(norm, nn.Identity) or (type(norm) is nn.LayerNorm and norm.elementwise_affine)
+    fused_rope = pos is None or isinstance(rope, RoPE2D)
+    if t.is_cuda and t.shape[-1] == 64 and fused_norm and fused_rope and not (isinstance(norm, nn.Identity) and pos is None):
+        cos = sin = None
+        if pos is not None:
+            n_pos = rope.max_positions or int(pos.max()) + 1
+            cos, sin = rope.tables(64, n_pos, t.device, t.dtype)
+        ln = norm if isinstance(norm, nn.LayerNorm) else None
+        out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
+                            ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
+        if out is not None:
+            return out
+    t = norm(t).to(t.dtype)
+    return rope(t, pos) if pos is not None else t
+
+
 class SparseFlashAttentionRope(nn.Module):
     def __init__(
         self,
@@ -66,24 +88,10 @@ class SparseFlashAttentionRope(nn.Module):
         self.topk = topk
         self.keep_topk_idx = False   # debugging aid: keep the last forward's block indices in ``last_topk_idx``
         self.last_topk_idx = None
+        self.last_path = None        # which route the last forward took: "fused-merge", "two-operators" or "autograd"
 
     def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
-        """qk-norm, cast and RoPE of one tensor: one fused kernel where it is built (head_dim 64, LayerNorm or no
-        norm, the package's RoPE2D), the separate torch modules otherwise.  Same rounding points either way."""
-        fused_norm = isinstance(norm, nn.Identity) or (type(norm) is nn.LayerNorm and norm.elementwise_affine)
-        fused_rope = pos is None or isinstance(self.rope, RoPE2D)
-        if t.shape[-1] == 64 and fused_norm and fused_rope and not (isinstance(norm, nn.Identity) and pos is None):
-            cos = sin = None
-            if pos is not None:
-                n_pos = self.rope.max_positions or int(pos.max()) + 1
-                cos, sin = self.rope.tables(64, n_pos, t.device, t.dtype)
-            ln = norm if isinstance(norm, nn.LayerNorm) else None
-            out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
-                                ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
-            if out is not None:
-                return out
-        t = norm(t).to(t.dtype)
-        return self.rope(t, pos) if pos is not None else t
+        return norm_rope_fused_or_eager(t, norm, self.rope, pos)
 
     def _forward_with_grad(self, x: Tensor, xpos: Optional[Tensor]) -> Tensor:
         """The same layer as a differentiable composition (training): the two attention operators carry their own
@@ -128,6 +136,7 @@ class SparseFlashAttentionRope(nn.Module):
 
     def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            self.last_path = "autograd"
             return self._forward_with_grad(x, xpos)
         b, n, c = x.shape
         h = self.num_heads
@@ -161,7 +170,9 @@ class SparseFlashAttentionRope(nn.Module):
             self.last_topk_idx = idx
 
         out = ops.select_attn_merge(q, k, v, idx, o_c, gate, block)
+        self.last_path = "fused-merge"
         if out is None:
+            self.last_path = "two-operators"
             out = ops.gated_merge(o_c, ops.select_attn(q, k, v, idx, block), gate, block)
 
         out = self.proj(out)

@@ -31,6 +31,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from ..layers import RoPE2D, SparseFlashAttentionRope
+from ..layers.sparse_attention import norm_rope_fused_or_eager
 from ..sparse_attn import ops
 
 
@@ -80,17 +81,7 @@ class DenseAttentionRope(nn.Module):
         self.rope = rope
 
     def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
-        if t.is_cuda and t.shape[-1] == 64 and (pos is not None or isinstance(norm, nn.LayerNorm)):
-            cos = sin = None
-            if pos is not None:
-                cos, sin = self.rope.tables(64, self.rope.max_positions or int(pos.max()) + 1, t.device, t.dtype)
-            ln = norm if isinstance(norm, nn.LayerNorm) else None
-            out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
-                                ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
-            if out is not None:
-                return out
-        t = norm(t).to(t.dtype)
-        return self.rope(t, pos) if pos is not None else t
+        return norm_rope_fused_or_eager(t, norm, self.rope, pos)
 
     def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
         b, n, c = x.shape
@@ -239,10 +230,14 @@ class Pi3SparseLike(nn.Module):
         reg = torch.zeros((self.register_token.shape[1], 2), dtype=patch.dtype, device=device)
         return torch.cat((reg, patch), dim=0)[None].expand(f, -1, -1).contiguous()
 
-    def forward(self, imgs: Tensor) -> dict:
-        """imgs [B, F, 3, H, W] in [0,1] -> dict(points, local_points, conf, camera_poses)."""
+    def forward(self, imgs: Tensor, return_features: bool = False) -> dict:
+        """imgs [B, F, 3, H, W] in [0,1] -> dict(points, local_points, conf, camera_poses); ``return_features`` adds the
+        decoder output the heads read (last frame-local and last global block, concatenated) under "features"."""
         b, f, _, hh, ww = imgs.shape
         gh, gw = hh // self.patch, ww // self.patch
+        # cos/sin tables of the fused norm/RoPE kernel sized for THIS call's grid (patch coordinates run 1..gh, 1..gw;
+        # the kernel clamps positions beyond its table, so a table sized at construction would be wrong for larger frames)
+        self.rope.max_positions = max(gh, gw) + 1
         x = ((imgs - self.image_mean) / self.image_std).reshape(b * f, 3, hh, ww).to(self.register_token.dtype)
         x = self.encoder(x)                                                        # [B*F, gh*gw, dim]
         x = torch.cat((self.register_token.expand(b * f, -1, -1), x), dim=1)       # [B*F, T, dim]
@@ -263,5 +258,8 @@ class Pi3SparseLike(nn.Module):
         local_points = torch.cat((xy * z, z), dim=-1).reshape(b, f, gh * self.patch, gw * self.patch, 3)
         homog = torch.cat((local_points, torch.ones_like(local_points[..., :1])), dim=-1)
         points = torch.einsum("bnij,bnhwj->bnhwi", poses, homog)[..., :3]
-        return dict(points=points, local_points=local_points,
-                    conf=conf.reshape(b, f, gh * self.patch, gw * self.patch, 1), camera_poses=poses)
+        out = dict(points=points, local_points=local_points,
+                   conf=conf.reshape(b, f, gh * self.patch, gw * self.patch, 1), camera_poses=poses)
+        if return_features:
+            out["features"] = feat
+        return out
