@@ -25,6 +25,11 @@ if str(ROOT) not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# (config, top-k, block, merge fused) -> HBM bytes per launch of the selection kernel and the profile summary they come from
+MEASURED_TRAFFIC = {
+    ("cfg3", 16, 64, True): (2.34e9, "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md"),
+    ("cfg4", 16, 64, True): (9.48e9, "profiles/layer_cfg4_1000f_bf16_kernel_stats.md"),
+}
 
 
 def parse_args():
@@ -335,8 +340,8 @@ def main() -> int:
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
             # HBM bytes per launch: not measured inside this run; the figure is the one rocprofv3 FETCH_SIZE / WRITE_SIZE
             # gave for this kernel on this workload, scaled by a plain copy (file named in traffic_source)
-            "traffic": 2.34e9 if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
-            "traffic_source": "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md" if (fused and args.config == "cfg3" and topk == 16 and block == 64) else None,
+            "traffic": MEASURED_TRAFFIC.get((args.config, topk, block, fused), (None, None))[0],
+            "traffic_source": MEASURED_TRAFFIC.get((args.config, topk, block, fused), (None, None))[1],
         },
     }
     if not args.no_cpu_baseline:
