@@ -8,8 +8,8 @@
  * (head_dim) stride of every q/k/v/o tensor is 1.  Launches are asynchronous on `stream`
  * (a hipStream_t passed as void*; NULL = the default stream).  Every function returns
  * S3R_OK or a negative error code and never throws; s3r_last_error() gives the message of
- * the calling thread's last failure.  No entry point allocates memory.  State kept between calls: the S3R_*
- * environment switches (read once, on first use) and the built-in score buffer of
+ * the calling thread's last failure.  No entry point allocates memory.  State kept between calls: the
+ * S3R_B16_KERNEL environment switch (read once, on first use) and the built-in score buffer of
  * s3r_compressed_attn_topk_static; nothing else.
  */
 #ifndef SPEED3R_HIP_H

@@ -151,29 +151,24 @@ static int select_attn_impl(const char* who, const void* q, const void* k, const
   p.scb = m.scb; p.sch = m.sch; p.scm = m.scm; p.sgb = m.sgb; p.sgh = m.sgh; p.sgn = m.sgn;
 
   const int es = elt_size(dtype);
-  // (row strides below 2^20 elements: the tile transfers use 32-bit byte offsets inside a 64-row tile)
+  // (row strides of q, k, v positive and below 2^20 elements: the transfers use 32-bit byte offsets inside a 64-row tile)
   const bool mfma_ok = dtype != S3R_F32 && D == 64 && block == 64 && K <= 64 && softmax_scale > 0.f &&
-                       skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
-                       vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
+                       skn > 0 && svn > 0 && sqn > 0 && skn < (1 << 20) && svn < (1 << 20) && sqn < (1 << 20) &&
+                       vec_ok(q, es, sqb, sqh, sqn) && vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
                        (merge ? (vec_ok(m.o_cmp, es, m.scb, m.sch, m.scm) && aligned16(m.out)) : vec_ok(o, es, sob, soh, son));
-  // default: the software-pipelined kernel; S3R_SELECT_KERNEL=basic picks the unpipelined one
-  static const bool basic = [] {
-    const char* e = getenv("S3R_SELECT_KERNEL");
-    return e != nullptr && strcmp(e, "basic") == 0;
-  }();
   // 16-token blocks (the reference layer's own setting): MFMA kernel that pairs query blocks
   const bool b16_ok = dtype != S3R_F32 && D == 64 && block == 16 && K <= 64 && softmax_scale > 0.f &&
-                      skn > 0 && svn > 0 && skn < (1 << 20) && svn < (1 << 20) && vec_ok(q, es, sqb, sqh, sqn) &&
-                      vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
+                      skn > 0 && svn > 0 && sqn > 0 && skn < (1 << 20) && svn < (1 << 20) && sqn < (1 << 20) &&
+                      vec_ok(q, es, sqb, sqh, sqn) && vec_ok(k, es, skb, skh, skn) && vec_ok(v, es, svb, svh, svn) &&
                       (merge ? (vec_ok(m.o_cmp, es, m.scb, m.sch, m.scm) && aligned16(m.out)) : vec_ok(o, es, sob, soh, son));
   if (merge) {
     if (b16_ok) return launch_select_b16(p, dtype, stream);
-    if (!mfma_ok || basic)
+    if (!mfma_ok)
       return fail(S3R_ERR_UNSUPPORTED, "%s: the fused merge needs an MFMA kernel (bf16/fp16, head_dim 64, block 64 or 16, "
                                        "16-byte aligned tensors); run s3r_select_attn and s3r_gated_merge instead", who);
     return launch_select_pipe(p, dtype, stream);
   }
-  if (mfma_ok) return basic ? launch_select_mfma(p, dtype, stream) : launch_select_pipe(p, dtype, stream);
+  if (mfma_ok) return launch_select_pipe(p, dtype, stream);
   if (b16_ok) return launch_select_b16(p, dtype, stream);
   return launch_attn_simple(p, dtype, /*select=*/true, stream);
 }

@@ -33,7 +33,6 @@ struct AttnParams {
 
 // launchers implemented in the .hip files; each returns S3R_OK or an error code
 int launch_attn_simple(const AttnParams& p, int dtype, bool select, void* stream);
-int launch_select_mfma(const AttnParams& p, int dtype, void* stream);
 int launch_select_pipe(const AttnParams& p, int dtype, void* stream);
 int launch_select_b16(const AttnParams& p, int dtype, void* stream);  // block 16
 int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream);

@@ -620,7 +620,7 @@ int launch_compressed_mfma(const AttnParams& p, int dtype, void* stream) {
     return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for Lk <= 2^21 and key strides < 2^24; pass a scores buffer");
   if (p.o != nullptr) {
     int rc;
-    if (p.Lq == p.Lk && p.skn < (1 << 20) && p.svn < (1 << 20)) {
+    if (p.Lq == p.Lk && p.sqm > 0 && p.skn > 0 && p.svn > 0 && p.sqm < (1 << 20) && p.skn < (1 << 20) && p.svn < (1 << 20)) {
       AttnParams d = p;
       d.idx = nullptr;  // dense sweep
       d.topk_idx = nullptr;

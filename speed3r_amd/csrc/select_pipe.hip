@@ -1,8 +1,29 @@
-// Selection-branch attention, software-pipelined variant (bf16 / fp16 I/O, block 64, head_dim 64).
+// Selection-branch attention on the gfx950 matrix cores (bf16 / fp16 I/O, block 64, head_dim 64), software-pipelined
+// inside the wave.
 //
-// Same roles as select_mfma.hip: one wavefront owns one 64-row query block of one head and walks the
-// block's selected key blocks, S^T = K Q^T and O^T += V^T P^T on v_mfma_f32_32x32x16, K and V tiles
-// through wave-private LDS, two waves per SIMD.  The difference is the order of work inside the wave.
+// One wavefront owns one 64-row query block of one head and walks that block's selected key blocks; the waves of a
+// workgroup take consecutive query blocks and never synchronise with each other (each has a private LDS region); two
+// waves per SIMD.
+//   * S^T = K Q^T with v_mfma_f32_32x32x16: the accumulator layout puts one QUERY per lane (column = lane & 31) and 16
+//     keys per 32x32 tile in its registers, so row maxima and row sums are in-lane loops plus one exchange with
+//     lane ^ 32.
+//   * P is rounded to the I/O dtype in registers; the accumulator layout of S^T is already the B-operand layout of
+//     O^T = V^T P^T (contraction index = key), with a fixed permutation of keys inside each group of 16 that the V
+//     operand simply follows.
+//   * K and V tiles go global -> LDS without passing through registers (buffer_load ... lds, 16 bytes per lane).  K
+//     fragments come back with ds_read_b128 (lane = key row; the 16-byte chunks of a row are stored XOR-swizzled by
+//     the row number so that the reads are conflict free), V^T fragments with ds_read_b64_tr_b16, which hands each
+//     lane 4 consecutive KEYS of one head_dim column: the A operand V^T without an explicit transpose (rows are 128
+//     bytes; the chunks of rows 2,3 (mod 4) are stored with their halves swapped so that the four rows one transposed
+//     read touches fall into four disjoint bank groups).
+//   * The softmax runs in base 2 on logits pre-multiplied by scale*log2(e); statistics are fp32.  Softmax is shift
+//     invariant: the loop uses ONE reference value per query row, the row maximum of the first half tile, and never
+//     rescales the accumulators; if a row sum ends above 2^100 or is not finite the query block is recomputed by an
+//     unpipelined stage with a true online softmax, which also handles every occurrence of the ragged last key block.
+//   * Workgroup -> work mapping is XCD-aware: hardware deals workgroups round-robin over the 8 XCDs, so workgroup w is
+//     given work item (w % 8) * per_xcd + w / 8: each XCD then walks a contiguous range of query blocks of one head at
+//     a time and its L2 sees one head's K/V.
+//
 // The unit of the pipeline is HALF a key tile (32 keys x 64 queries): its S^T is 8 MFMAs, its PV is 8
 // MFMAs, its softmax is 32 exponentials per lane.  In one phase the wave issues
 //
@@ -19,9 +40,6 @@
 // compiler then knows that a read of one does not depend on a transfer into another).  A half
 // buffer is refilled (buffer_load ... lds, 16 bytes per lane) right after its fragments have been read,
 // two phases before it is needed again.
-//
-// Softmax reference, overflow fallback, ragged last key block, register layouts and the LDS swizzles are
-// those of select_mfma.hip.
 #include "select_common.h"
 #include "attn_params.h"
 

@@ -79,6 +79,10 @@ def pool_qkv_packed(qkv: torch.Tensor, num_heads: int, block: int) -> Tuple[torc
     return y[:, :num_heads], y[:, num_heads:2 * num_heads], y[:, 2 * num_heads:]
 
 
+# largest fp32 score buffer compressed_attn_topk allocates for its own use (a caller that asks for the scores gets them whole)
+SCORE_BUFFER_BYTES = 1 << 30
+
+
 def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], topk: Optional[int],
                          softmax_scale: Optional[float] = None, return_scores: bool = False,
                          return_lse: bool = False, materialize_scores: Optional[bool] = None,
@@ -124,19 +128,38 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Ten
         bool(topk) and materialize_scores is None and not fused_ok)
     if materialize_scores is False and topk and not fused_ok:
         raise RuntimeError("fused top-k is not available for this dtype/shape; allow a score buffer")
-    scores = torch.empty((b, h, lq, lk), dtype=torch.float32, device=q.device) if want_scores else None
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=q.device) if return_lse else None
-    with torch.cuda.device(q.device):
-        rc = _lib.lib().s3r_compressed_attn_topk(
-            q.data_ptr(), k.data_ptr(), None if indices_only else v.data_ptr(), None if indices_only else o.data_ptr(),
-            lse.data_ptr() if lse is not None else None,
-            idx.data_ptr() if idx is not None else None,
-            scores.data_ptr() if scores is not None else None,
-            b, h, lq, lk, d, topk or 0,
-            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            v.stride(0), v.stride(1), v.stride(2), *((0, 0, 0) if indices_only else (o.stride(0), o.stride(1), o.stride(2))),
-            scale, _code(q), _stream(q))
-    _lib.check(rc, "s3r_compressed_attn_topk")
+    st3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+
+    def launch(q_, o_, lse_, idx_, scores_, rows):
+        with torch.cuda.device(q.device):
+            rc = _lib.lib().s3r_compressed_attn_topk(
+                q_.data_ptr(), k.data_ptr(), None if indices_only else v.data_ptr(), None if indices_only else o_.data_ptr(),
+                lse_.data_ptr() if lse_ is not None else None,
+                idx_.data_ptr() if idx_ is not None else None,
+                scores_.data_ptr() if scores_ is not None else None,
+                b, h, rows, lk, d, topk or 0, *st3(q_), *st3(k), *st3(v),
+                *((0, 0, 0) if indices_only else st3(o_)), scale, _code(q), _stream(q))
+        _lib.check(rc, "s3r_compressed_attn_topk")
+
+    rows_per_pass = max(128, (SCORE_BUFFER_BYTES // (4 * b * h * lk)) // 128 * 128)
+    if want_scores and not return_scores and lq > rows_per_pass:
+        # top-k values without a fused kernel (fp32, top-k 64, ...) on many pooled tokens: the score buffer holds a
+        # band of query rows at a time instead of the whole [Lq, Lk] matrix (16.9 GB at a million tokens)
+        scores = torch.empty((b, h, rows_per_pass, lk), dtype=torch.float32, device=q.device)
+        for r0 in range(0, lq, rows_per_pass):
+            r1 = min(lq, r0 + rows_per_pass)
+            idx_c = torch.empty((b, h, r1 - r0, topk), dtype=torch.int32, device=q.device) if topk else None
+            lse_c = torch.empty((b, h, r1 - r0), dtype=torch.float32, device=q.device) if return_lse else None
+            launch(q[:, :, r0:r1], o[:, :, r0:r1], lse_c, idx_c, scores, r1 - r0)
+            if idx_c is not None:
+                idx[:, :, r0:r1] = idx_c
+            if lse_c is not None:
+                lse[:, :, r0:r1] = lse_c
+        scores = None
+    else:
+        scores = torch.empty((b, h, lq, lk), dtype=torch.float32, device=q.device) if want_scores else None
+        launch(q, o, lse, idx, scores, lq)
     out = [o, idx]
     if return_scores:
         out.append(scores)
@@ -494,10 +517,11 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
     return _SIDE_STREAMS[key]
 
 
-def _two_kernel_compressed(q: torch.Tensor, topk: int) -> bool:
-    """True where the compressed branch is two independent kernels (attention, indices without a score buffer)."""
+def _two_kernel_compressed(q: torch.Tensor, topk: int, block: int = 1) -> bool:
+    """True where the compressed branch is two independent kernels (attention, indices without a score buffer).
+    ``q``: the pooled queries (``block`` = 1) or the full tokens that will be pooled over ``block`` tokens."""
     return (q.dtype != torch.float32 and q.shape[-1] == 64 and topk in (1, 2, 4, 8, 16, 32)
-            and q.shape[2] <= (1 << 21) * 64 and _lib.lib_has_fused_topk())
+            and -(-q.shape[2] // block) <= (1 << 21) and _lib.lib_has_fused_topk())
 
 
 def topk_indices_on_side_stream(qc: torch.Tensor, kc: torch.Tensor, topk: int, softmax_scale: Optional[float] = None):
@@ -546,7 +570,7 @@ def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g
             timeline[name] = ev
 
     mark("start")
-    if overlap and materialize_scores is not True and _two_kernel_compressed(q, topk) and q.is_cuda:
+    if overlap and materialize_scores is not True and _two_kernel_compressed(q, topk, block) and q.is_cuda:
         qc, kc = pool_mean(q, block), pool_mean(k, block)
         idx, join = topk_indices_on_side_stream(qc, kc, topk, softmax_scale)
         vc = pool_mean(v, block)
