@@ -53,7 +53,7 @@ def parse_args():
                     help="run the index kernel on a second stream beside the pooling of v and the compressed attention")
     ap.add_argument("--backward", action="store_true",
                     help="time the backward of the two attention operators (one JSON line of its own; not the headline metric)")
-    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "copy"],
+    ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "prepass", "copy"],
                     help="profiling aid: after one full pass, launch only this stage `steps` times (no JSON line)")
     return ap.parse_args()
 
@@ -94,6 +94,26 @@ def cpu_baseline(q, k, v, gate, block, topk, heads):
         "sample": f"oracle (eager fp32 PyTorch + numpy top-k) on heads 0..{heads - 1} of {total_heads}, all tokens: "
                   f"{dt:.2f} s measured, scaled x{total_heads // heads} to the full layer",
     }
+
+
+def _prepass_stage(qd, kd, vd, block):
+    """The layer's one-pass kernel over a packed [1, N, 3*H*64] projection built from the workload's q, k, v: block
+    means of the raw rows + LayerNorm + RoPE2D of q and k (positions of a 37 x 28 patch grid after 5 register tokens)."""
+    import torch
+
+    from speed3r_amd.layers import RoPE2D
+    from speed3r_amd.sparse_attn import ops
+
+    _, h, n, d = qd.shape
+    packed = torch.stack((qd[0], kd[0], vd[0]), dim=0).permute(2, 0, 1, 3).reshape(1, n, 3 * h * d).contiguous()
+    t = torch.arange(n, device=qd.device) % 1041
+    patch = (t - 5).clamp(min=0)
+    pos = torch.where((t >= 5)[:, None], torch.stack((patch // 28 + 1, patch % 28 + 1), dim=-1), torch.zeros_like(t)[:, None])[None]
+    cos, sin = RoPE2D(100.0).tables(64, 39, qd.device, qd.dtype)
+    g = torch.Generator().manual_seed(9)
+    ln = [((1 + 0.1 * torch.randn(64, generator=g)).to(qd.dtype).to(qd.device), (0.1 * torch.randn(64, generator=g)).to(qd.dtype).to(qd.device))
+          for _ in range(2)]
+    return lambda: ops.qkv_prepass(packed, h, block, pos, cos, sin, ln[0], ln[1], 1e-6)
 
 
 def run_end_to_end(args) -> int:
@@ -262,6 +282,7 @@ def main() -> int:
                 "select_merge": lambda: s3r.select_attn_merge(qd, kd, vd, idx, o_cmp, gd, block),
                 # a plain device copy of q (reads and writes q.nbytes): the yardstick for the HBM byte counters
                 "copy": lambda: torch.empty_like(qd).copy_(qd),
+                "prepass": _prepass_stage(qd, kd, vd, block),
             }[args.only]
             torch.cuda.synchronize()
             t0 = time.perf_counter()

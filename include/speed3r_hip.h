@@ -181,6 +181,25 @@ int s3r_norm_rope(const void* x, void* y, const int32_t* pos, const void* cos_ta
                   int dtype, void* stream);
 
 /*
+ * The layer's pre-pass over the packed q/k/v projection in ONE kernel: block means of the raw q, k, v rows (the
+ * compressed branch's inputs) and qk-LayerNorm + 2-D rotary embedding of the full-token q and k, each input row read once.
+ * Replaces F.avg_pool1d on the raw projection, the three .contiguous() copies, q_norm / k_norm with their casts and
+ * the two rope calls on the full tokens (pi3/models/layers/sparse_attention.py:97-99,115-124).  Same bits as
+ * s3r_pool_mean on q, k, v followed by s3r_norm_rope on q and k.
+ *   q, k, v: [B,H,N,64] views with common strides sxb,sxh,sxn (last stride 1), e.g. the three sections of the packed
+ *     [B,N,3*H*64] projection; v is only read (the attention kernels take it in place).
+ *   q_out, k_out: contiguous [B,H,N,64];  qc, kc, vc: contiguous [B,H,ceil(N/block),64] (a ragged last block is a mean
+ *     over its valid tokens).
+ *   pos, cos_tab, sin_tab, P, eps and the LayerNorm parameters (qn_* for q, kn_* for k; both NULL for no norm) as in
+ *     s3r_norm_rope.
+ */
+int s3r_qkv_prepass(const void* q, const void* k, const void* v, void* q_out, void* k_out, void* qc, void* kc, void* vc,
+                    const int32_t* pos, const void* cos_tab, const void* sin_tab, int P,
+                    const void* qn_w, const void* qn_b, const void* kn_w, const void* kn_b, float eps,
+                    int B, int H, int64_t N, int D, int block,
+                    int64_t sxb, int64_t sxh, int64_t sxn, int64_t spb, int64_t spn, int dtype, void* stream);
+
+/*
  * LayerNorm over the channels of token rows:  y[r,:] = (x[r,:] - mean_r) * rstd_r * w + b, fp32 statistics, one
  * rounding to the I/O dtype.  Replaces, for inference, the nn.LayerNorm modules in front of the attention layers and
  * the MLPs (norm1 / norm2, pi3/models/layers/block.py:281,296,312,315).

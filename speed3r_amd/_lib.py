@@ -37,6 +37,8 @@ SIGNATURES = {
                                       *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
     "s3r_norm_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
                               c_int, c_int, c_int64, c_int, *_i64x3, c_int64, c_int64, c_int, c_void_p]),
+    "s3r_qkv_prepass": (c_int, [c_void_p] * 8 + [c_void_p, c_void_p, c_void_p, c_int] + [c_void_p] * 4 + [c_float, c_int, c_int, c_int64,
+                                c_int, c_int, *_i64x3, c_int64, c_int64, c_int, c_void_p]),
     "s3r_layer_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int64, c_int64, c_int, c_void_p]),
     "s3r_gated_merge": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int,
                                 *_i64x3, *_i64x3, *_i64x3, c_int, c_void_p]),

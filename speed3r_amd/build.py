@@ -13,7 +13,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / "csrc"
 LIB_NAME = "libspeed3r_hip.so"
-SOURCES = ["api.hip", "pool_merge.hip", "topk.hip", "attn_simple.hip", "select_pipe.hip", "compressed_mfma.hip", "norm_rope.hip", "layer_norm.hip", "attn_bwd.hip", "select_b16.hip", "key_lists.hip"]
+SOURCES = ["api.hip", "pool_merge.hip", "topk.hip", "attn_simple.hip", "select_pipe.hip", "compressed_mfma.hip", "norm_rope.hip", "qkv_prepass.hip", "layer_norm.hip", "attn_bwd.hip", "select_b16.hip", "key_lists.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

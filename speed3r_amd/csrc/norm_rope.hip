@@ -44,14 +44,12 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < VEC; i++) s += v[i];
-#pragma unroll
-    for (int off = 1; off < LPR; off <<= 1) s += __shfl_xor(s, off);
+    s = group_sum<LPR>(s);
     const float mean = s * (1.0f / D);
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < VEC; i++) q += (v[i] - mean) * (v[i] - mean);
-#pragma unroll
-    for (int off = 1; off < LPR; off <<= 1) q += __shfl_xor(q, off);
+    q = group_sum<LPR>(q);
     const float rstd = 1.0f / sqrtf(q * (1.0f / D) + eps);
     uint4 wr = *reinterpret_cast<const uint4*>(ln_w + lr * VEC);
     const T* we = reinterpret_cast<const T*>(&wr);
@@ -74,7 +72,7 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(
     const T* se = reinterpret_cast<const T*>(&sr);
 #pragma unroll
     for (int i = 0; i < VEC; i++) {
-      const float other = __shfl_xor(v[i], QL);                 // the paired value, one quarter away
+      const float other = lane_xor<QL>(v[i]);                 // the paired value, one quarter away
       const float rot = second ? other : -other;                // "rotate half": (-second quarter, first quarter)
       const float a = round_to<T>(v[i] * to_f32(ce[i]));
       const float c2 = round_to<T>(rot * to_f32(se[i]));

@@ -66,4 +66,25 @@ __device__ __forceinline__ uint32_t sortable_key(float s) {
 
 constexpr int kWave = 64;
 
+// Value held by lane ^ MASK.  Masks 1 and 2 stay inside a quad and ride on the DPP operand path of an ordinary move
+// (no LDS crossbar); masks up to 16 use the swizzle unit without an address register; larger ones the general permute.
+template <int MASK> __device__ __forceinline__ float lane_xor(float x) {
+  static_assert(MASK > 0 && MASK < 64 && (MASK & (MASK - 1)) == 0, "one bit of the lane number");
+  const int v = __float_as_int(x);
+  if constexpr (MASK == 1) return __int_as_float(__builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false));       // quad_perm [1,0,3,2]
+  else if constexpr (MASK == 2) return __int_as_float(__builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false));  // quad_perm [2,3,0,1]
+  else if constexpr (MASK < 32) return __int_as_float(__builtin_amdgcn_ds_swizzle(v, (MASK << 10) | 0x1F));       // bit mode: and 0x1f, xor MASK
+  else return __shfl_xor(x, MASK);
+}
+// sum over the aligned group of N lanes (a power of two) the lane belongs to
+template <int N> __device__ __forceinline__ float group_sum(float s) {
+  if constexpr (N >= 2) s += lane_xor<1>(s);
+  if constexpr (N >= 4) s += lane_xor<2>(s);
+  if constexpr (N >= 8) s += lane_xor<4>(s);
+  if constexpr (N >= 16) s += lane_xor<8>(s);
+  if constexpr (N >= 32) s += lane_xor<16>(s);
+  if constexpr (N >= 64) s += lane_xor<32>(s);
+  return s;
+}
+
 }  // namespace s3r

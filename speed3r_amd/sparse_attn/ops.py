@@ -292,6 +292,53 @@ def norm_rope(x: torch.Tensor, positions: Optional[torch.Tensor], cos_tab: Optio
     return y
 
 
+def qkv_prepass(qkv: torch.Tensor, num_heads: int, block: int, positions: Optional[torch.Tensor],
+                cos_tab: Optional[torch.Tensor], sin_tab: Optional[torch.Tensor],
+                q_ln: Optional[Tuple[torch.Tensor, Optional[torch.Tensor]]] = None,
+                k_ln: Optional[Tuple[torch.Tensor, Optional[torch.Tensor]]] = None, eps: float = 1e-5):
+    """The layer's pre-pass over the packed projection ``[B, N, 3*H*64]`` (layout ``(qkv h d)``) in one kernel:
+    returns ``(q, k, v, q_c, k_c, v_c)`` -- q, k ``[B,H,N,64]`` contiguous after LayerNorm (``q_ln``/``k_ln`` = (weight,
+    bias) or None) and RoPE2D at ``positions`` (None: no rotation), v the strided view of the projection, and the
+    block means of the RAW q, k, v ``[B,H,ceil(N/block),64]``.  Same bits as :func:`pool_qkv_packed` followed by
+    :func:`norm_rope` on q and k.  Returns None when the library has no kernel for the shape (head_dim other than 64)."""
+    _need_device(qkv)
+    _forward_only(qkv)
+    b, n, c3 = qkv.shape
+    d = c3 // (3 * num_heads)
+    if d != 64 or c3 != 3 * num_heads * 64 or qkv.stride(-1) != 1:
+        return None
+    assert (q_ln is None) == (k_ln is None), "q and k are normalised together or not at all"
+    h = num_heads
+    q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)   # each [B,H,N,D], common strides
+    nc = -(-n // block)
+    q_out, k_out = (torch.empty((b, h, n, d), dtype=qkv.dtype, device=qkv.device) for _ in range(2))
+    qc, kc, vc = (torch.empty((b, h, nc, d), dtype=qkv.dtype, device=qkv.device) for _ in range(3))
+    pos32 = None
+    p = 0
+    if positions is not None:
+        assert positions.shape == (b, n, 2), f"positions shape {tuple(positions.shape)} != {(b, n, 2)}"
+        assert cos_tab is not None and sin_tab is not None and cos_tab.shape == sin_tab.shape and cos_tab.shape[1] == 16
+        assert cos_tab.dtype == qkv.dtype and sin_tab.dtype == qkv.dtype, "tables must have the tokens' dtype"
+        pos32 = positions.to(device=qkv.device, dtype=torch.int32).contiguous()
+        cos_tab, sin_tab = cos_tab.contiguous(), sin_tab.contiguous()
+        p = cos_tab.shape[0]
+
+    def par(t):
+        return t.detach().to(qkv.dtype).contiguous() if t is not None else None
+
+    qw, qb = (par(q_ln[0]), par(q_ln[1])) if q_ln is not None else (None, None)
+    kw, kb = (par(k_ln[0]), par(k_ln[1])) if k_ln is not None else (None, None)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(qkv.device):
+        rc = _lib.lib().s3r_qkv_prepass(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), k_out.data_ptr(), qc.data_ptr(), kc.data_ptr(),
+            vc.data_ptr(), ptr(pos32), ptr(cos_tab) if pos32 is not None else None, ptr(sin_tab) if pos32 is not None else None, p,
+            ptr(qw), ptr(qb), ptr(kw), ptr(kb), float(eps), b, h, n, d, block, q.stride(0), q.stride(1), q.stride(2),
+            pos32.stride(0) if pos32 is not None else 0, pos32.stride(1) if pos32 is not None else 0, _code(qkv), _stream(qkv))
+    _lib.check(rc, "s3r_qkv_prepass")
+    return q_out, k_out, v, qc, kc, vc
+
+
 def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> Optional[torch.Tensor]:
     """``F.layer_norm(x, (C,), weight, bias, eps)`` over the last dimension of token rows in one pass (inference).
 

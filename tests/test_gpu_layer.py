@@ -145,3 +145,46 @@ def test_layer_gradients_match_autograd_through_the_oracle(n, block_size, topk):
     for k in want:
         tol = 5e-2 * max(1.0, float(want[k].abs().max()))
         assert max_abs(got[k], want[k]) <= tol, (k, max_abs(got[k], want[k]), tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("n,block,with_norm,with_pos", [(320, 64, True, True), (200, 64, True, True), (1041, 16, True, True),
+                                                        (77, 16, False, True), (130, 64, True, False), (5, 64, True, True)])
+def test_one_pass_over_the_packed_projection_equals_pooling_then_norm_rope(dtype, n, block, with_norm, with_pos):
+    """s3r_qkv_prepass (block means of raw q, k, v + LayerNorm + RoPE of q and k in one pass) against s3r_pool_mean on
+    the packed projection followed by s3r_norm_rope on q and k: the same bits, ragged last blocks included."""
+    from speed3r_amd.sparse_attn import ops
+    b, h = 2, 3
+    g = torch.Generator().manual_seed(n + block)
+    qkv = (torch.randn((b, n, 3 * h * 64), generator=g) * 0.7).to(dtype).to(DEV)
+    pos = torch.randint(0, 40, (b, n, 2), generator=g).to(DEV) if with_pos else None
+    rope = RoPE2D(freq=100.0)
+    cos, sin = rope.tables(64, 40, DEV, dtype) if with_pos else (None, None)
+    lnq = ((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV), (0.2 * torch.randn(64, generator=g)).to(dtype).to(DEV))
+    lnk = ((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV), None)
+    got = ops.qkv_prepass(qkv, h, block, pos, cos, sin, lnq if with_norm else None, lnk if with_norm else None, 1e-6)
+    q, k, v = qkv.view(b, n, 3, h, 64).permute(2, 0, 3, 1, 4).unbind(0)
+    want_c = ops.pool_qkv_packed(qkv, h, block)
+    want_q = ops.norm_rope(q, pos, cos, sin, lnq[0] if with_norm else None, lnq[1] if with_norm else None, 1e-6)
+    want_k = ops.norm_rope(k, pos, cos, sin, lnk[0] if with_norm else None, None, 1e-6)
+    assert torch.equal(got[0], want_q) and torch.equal(got[1], want_k)
+    assert got[2].data_ptr() == v.data_ptr() and got[2].stride() == v.stride()
+    for a, w in zip(got[3:], want_c):
+        assert a.shape == (b, h, -(-n // block), 64) and torch.equal(a, w)
+
+
+def test_layer_takes_the_one_pass_route_where_it_is_built():
+    torch.manual_seed(11)
+    m = SparseFlashAttentionRope(dim=128, num_heads=2, qkv_bias=True, qk_norm=True, rope=RoPE2D(100.0), block_size=8, topk=2)
+    m = m.to(torch.bfloat16).to(DEV).eval()
+    x = torch.randn(1, 200, 128, device=DEV).to(torch.bfloat16)
+    pos = torch.randint(0, 30, (1, 200, 2), device=DEV)
+    with torch.no_grad():
+        m(x, xpos=pos)
+        assert m.last_prepass is True and m.last_path == "fused-merge"
+        m2 = SparseFlashAttentionRope(dim=128, num_heads=2, block_size=8, topk=2).to(torch.bfloat16).to(DEV).eval()
+        m2(x)                                   # no norm, no positions: nothing to do to q and k, no pre-pass
+        assert m2.last_prepass is False
+        m3 = SparseFlashAttentionRope(dim=128, num_heads=2, qk_norm=True, rope=RoPE2D(100.0), block_size=4, topk=4).to(torch.bfloat16).to(DEV).eval()
+        m3(x, xpos=pos)                         # 16-token blocks: separate kernels, the index kernel starts earlier
+        assert m3.last_prepass is False and m3.last_path == "fused-merge"
