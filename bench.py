@@ -49,8 +49,9 @@ def parse_args():
     ap.add_argument("--cpu-heads", type=int, default=16, help="heads of the workload the CPU baseline runs")
     ap.add_argument("--materialize-scores", action="store_true", help="force the two-kernel score/top-k path")
     ap.add_argument("--no-fuse-merge", action="store_true", help="run selection attention and the gated merge as two kernels")
-    ap.add_argument("--overlap", action="store_true",
-                    help="run the index kernel on a second stream beside the pooling of v and the compressed attention")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="run every kernel on one stream (per-kernel times for pooling and the compressed branch); by default "
+                         "the index kernel runs on a second stream beside the pooling of v and the compressed attention")
     ap.add_argument("--backward", action="store_true",
                     help="time the backward of the two attention operators (one JSON line of its own; not the headline metric)")
     ap.add_argument("--only", default=None, choices=["pool", "compressed_topk", "select", "merge", "select_merge", "prepass", "copy"],
@@ -260,7 +261,7 @@ def main() -> int:
     mat = True if args.materialize_scores else None
 
     fused = not args.no_fuse_merge
-    overlap = args.overlap and not args.materialize_scores
+    overlap = not args.no_overlap and not args.materialize_scores and cfg.dtype != torch.float32 and topk in (1, 2, 4, 8, 16, 32)
 
     def step(timeline=None):
         return s3r.sparse_global_attention(qd, kd, vd, gd, block, topk, materialize_scores=mat, fuse_merge=fused,

@@ -595,17 +595,18 @@ def topk_indices_on_side_stream(qc: torch.Tensor, kc: torch.Tensor, topk: int, s
 def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
                             block: int = 64, topk: int = 16, softmax_scale: Optional[float] = None,
                             return_parts: bool = False, materialize_scores: Optional[bool] = None,
-                            fuse_merge: bool = True, overlap: bool = False, timeline: Optional[dict] = None):
+                            fuse_merge: bool = True, overlap: Optional[bool] = None, timeline: Optional[dict] = None):
     """The whole path on post-norm/RoPE q, k, v ``[B,H,N,D]`` and gate ``[B,H,N,2]``:
     pool -> compressed attention + top-k -> selection attention -> gated merge -> ``[B,N,H*D]``.
     The merge runs in the selection kernel's epilogue where the library offers it (same bits either way);
     ``return_parts`` needs the selection output and therefore runs the two operators separately.
 
-    ``overlap``: the indices need pooled q and k only, the compressed attention output is not read before the
-    merge.  Where the two come from different kernels, the index kernel runs on a second stream next to the
-    pooling of v and the compressed attention (same kernels, same results; only the schedule differs).  Measured at
-    266 496 tokens this schedule gains nothing here (the kernels fill the chip one by one), so it is off by default;
-    the layer module uses the same mechanism to hide the index kernel behind the HBM-bound norm/RoPE of the full tokens.
+    ``overlap`` (default: on where it applies): the indices need pooled q and k only, the compressed attention output
+    is not read before the merge.  Where the two come from different kernels (no score buffer), the index kernel runs
+    on a second stream next to the pooling of v and the compressed attention (same kernels, same results; only the
+    schedule differs).  The index kernel alone leaves most of the chip idle below a few thousand pooled tokens (one
+    workgroup per 128 pooled rows and head); measured at 266 496 tokens: 0.51 against 0.55 ms for everything in front
+    of the selection kernel.  ``overlap=False`` runs the kernels one after the other on the calling stream.
 
     ``timeline``: a dict that receives timing events of the calling stream under "start", "pooled" (sequential
     schedule only), "select" (everything before the selection kernel is done) and "end".
@@ -617,7 +618,8 @@ def sparse_global_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g
             timeline[name] = ev
 
     mark("start")
-    if overlap and materialize_scores is not True and _two_kernel_compressed(q, topk, block) and q.is_cuda:
+    if overlap is not False and materialize_scores is not True and not return_parts and q.is_cuda \
+            and _two_kernel_compressed(q, topk, block):
         qc, kc = pool_mean(q, block), pool_mean(k, block)
         idx, join = topk_indices_on_side_stream(qc, kc, topk, softmax_scale)
         vc = pool_mean(v, block)
