@@ -499,6 +499,14 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
                 const float settled = fmaxf(st[g / (16 / kGroup)][0], st[g / (16 / kGroup)][15]);
                 asm volatile("" ::"v"(settled));
               }
+              {  // No survivor among the group's 4 x 64 scores (NaNs of masked keys drop out of the maxima): next group, for
+                 // two maxima, one compare and one branch instead of four of each.  With K wanted out of several thousand keys,
+                 // three groups in four end here (16 266 keys, top-16: 1.11 -> 0.92 ms; 4 164 keys: 0.166 -> 0.152 ms); a
+                 // second test over eight registers in front of this one gains 2 % more and is not worth its code.
+                const int kt = g / (16 / kGroup), r = (g % (16 / kGroup)) * kGroup;
+                const float m4 = fmaxf(fmaxf(st[kt][r], st[kt][r + 1]), fmaxf(st[kt][r + 2], st[kt][r + 3]));
+                if (__builtin_amdgcn_ballot_w64(m4 >= thr) == 0) continue;
+              }
 #pragma unroll
               for (int e8 = 0; e8 < kGroup; e8++) {
                 const int kt = g / (16 / kGroup), r = (g % (16 / kGroup)) * kGroup + e8;
