@@ -3,16 +3,16 @@
 // (pi3/models/layers/sparse_attention.py:73,98,125; kernel topk_blocksparse_attention.py:35-128).
 //
 // One wavefront owns four consecutive query blocks (64 queries) of one head; one wave per workgroup.
-// The 32x32x16 MFMA wants 32 keys and 32 queries per tile, a query block has only 16 of each per list entry, so a
-// tile pairs TWO query blocks with ONE list entry of each: rows 0-15 of the key half tile hold the block the first
-// query block lists at position i, rows 16-31 the block the second one lists at position i.  S^T = K Q^T then has
-// two useful 16x16 quadrants (first block's keys x first block's queries, second x second); the other two are
-// masked to probability zero.  Half of the matrix work is thrown away, which is affordable: this shape is bound by
-// the texture path (a 2 KB key block serves 16 queries, a quarter of the reuse of the 64-token case), not by MFMA.
+// The 32x32x16 MFMA wants 32 keys and 32 queries per tile, a list entry offers 16 keys for 16 queries.  Two walks:
+//  * union walk (default): the wave walks the UNION of its four lists, two distinct key blocks per tile, all 64
+//    queries scored against both (neighbouring query blocks list mostly the same blocks, so most quadrants are
+//    useful); walk list built first, then a software pipeline over (tile, query half) units, see the kernel body;
+//  * pair walk (S3R_B16_KERNEL=pairs, cross-check, and tensors beyond 4 GB per head): a tile pairs TWO query blocks
+//    with ONE list entry of each, rows 0-15 of the key half tile hold the block the first query block lists at
+//    position i, rows 16-31 the block the second one lists at position i; S^T = K Q^T then has two useful 16x16
+//    quadrants, the other two are masked to probability zero; online softmax on the 8 own registers.
 // Everything else follows the 64-token kernels: one query per lane (S^T accumulator), P rounded to the I/O dtype,
-// O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16, K/V half tiles by direct transfers with explicit waits,
-// double buffered (the two query-block pairs of the wave alternate, so pair 1's tiles fly while pair 0 computes).
-// The softmax is online (running maximum per query, accumulators rescaled only when some maximum moved).
+// O^T += V^T P^T with V^T fragments from ds_read_b64_tr_b16, K/V half tiles by direct transfers with explicit waits.
 // Entries < 0 or starting at or beyond N are skipped, keys beyond N in the ragged last block are masked, a query
 // block with no valid entry gives zeros; up to 64 entries per query block.
 #include "select_common.h"
@@ -30,7 +30,7 @@ constexpr int kHalfBytes = 32 * 128;
 #endif
 // wavefronts (groups of four query blocks) per workgroup; the waves do not interact.  One: the unions differ in size
 // (cfg-3-like lists: 32 to 127 distinct blocks), and a workgroup keeps its slots until its slowest wave is done
-// (4 waves: 1.71 ms, 2: 1.50 ms, 1: 1.42 ms at 266 496 tokens, top-32).
+// (measured on the walk before the pipeline: 4 waves 1.71 ms, 2: 1.50 ms, 1: 1.42 ms at 266 496 tokens, top-32).
 constexpr int kWaves = S3R_B16_WAVES;
 constexpr float kLog2e = 1.4426950408889634f;
 typedef std::integral_constant<int, 0> H0;
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kWaves * kHalfBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kWaves * kHalfBytes];
 
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = kWaves == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int hh = lane >> 5;
   const int c = lane & 31;
@@ -229,61 +229,125 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
   if constexpr (UNION) {
     // Neighbouring query blocks list mostly the same key blocks.  The wave therefore walks the UNION of its four
     // lists: a tile is two distinct key blocks A, B (rows 0-15, 16-31), fetched once, and every one of the 64 queries
-    // whose block lists A (B) uses its 16 scores against A (B); cnt bytes say how often query block j lists the
-    // block (0: not at all, its scores are masked; above 1: a duplicated entry, the probabilities count that often).
-    // The visiting order differs from the lists' order, which changes fp32 summation order only.
-    uint64_t rem[4];
-    bool exact = false;  // second walk: running maximum
-    auto pop = [&](int32_t& blk, uint32_t& cnts) {  // next distinct key block and its four multiplicities, or -1
-      blk = -1;
-      cnts = 0;
+    // whose block lists A (B) uses its 16 scores against A (B).  The visiting order differs from the lists' order,
+    // which changes fp32 summation order only.
+    //
+    // 1. The walk list is built first, in registers: entry n (lane n & 63 of register n >> 6) holds a distinct block
+    //    and four count bytes (how often query block j lists it; 0: not at all, above 1: a duplicated entry, which
+    //    attends the block that often).  One step takes the first remaining entry of any list (one ballot, three
+    //    selects), removes the block from all four lists and counts it (four compares).
+    // 2. A software pipeline over units (tile t, half h of the 64 queries) then walks the list.  While the
+    //    exponentials of unit u run on the VALU, the matrix pipe takes the scores of unit u + 1 and the PV product of
+    //    unit u - 1, one MFMA per two exponentials.  K and V tiles come by direct transfers into two half buffers
+    //    each, 1.5 tile times ahead of their use; all buffer choices are static (the loop is written for even and odd
+    //    tiles), so that the only waits for transfers are the explicit ones.
+    __shared__ __attribute__((aligned(16))) int2 lds_walk[kWaves][264];  // up to 4 x 64 entries and the end mark
+    int2* const walk = lds_walk[wave];
+    const int32_t ragged_blk = (N & 15) ? (int32_t)(N >> 4) : -2;  // the block that ends before its 16th row ...
+    const int ragged_last = (int)(N & 15) - 1;
+    uint32_t ragged_cnts = 0;  // ... stays out of the list: it gets a step of its own after the pipeline
+    int n_union = 0;
+    uint32_t cnt_bits = 0;
+    {
+      bool alive[4];
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (blk < 0 && rem[j] != 0) blk = __builtin_amdgcn_readlane(my_idx[j], __ffsll((unsigned long long)rem[j]) - 1);
-      if (blk >= 0) {
+      for (int j = 0; j < 4; j++) alive[j] = my_idx[j] >= 0;
+      while (true) {
+        const uint64_t any = __ballot(alive[0] || alive[1] || alive[2] || alive[3]);
+        if (any == 0) break;
+        const int i = __ffsll((unsigned long long)any) - 1;
+        const int32_t front = alive[0] ? my_idx[0] : alive[1] ? my_idx[1] : alive[2] ? my_idx[2] : my_idx[3];
+        const int32_t blk = __builtin_amdgcn_readlane(front, i);
+        uint32_t cnts = 0;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const uint64_t hit = __ballot(my_idx[j] == blk) & rem[j];
-          rem[j] &= ~hit;
-          cnts |= (uint32_t)__popcll(hit) << (8 * j);
+        for (int j = 0; j < 4; j++) {  // entries equal to blk are all still there: a block leaves all lists at once
+          const bool hit = my_idx[j] == blk;
+          cnts |= (uint32_t)__popcll(__ballot(hit)) << (8 * j);
+          alive[j] = alive[j] && !hit;
+        }
+        cnt_bits |= cnts;
+        if (blk == ragged_blk) {
+          ragged_cnts = cnts;
+        } else {
+          walk[n_union] = make_int2(blk, (int32_t)cnts);  // every lane writes the same pair
+          n_union++;
         }
       }
+      walk[n_union] = make_int2(-1, 0);
+    }
+    const bool dup = (cnt_bits & 0xfefefefeu) != 0;  // some list names a block more than once (wave-uniform)
+    // tile tau = entries 2 tau, 2 tau + 1 of the walk list (-1 / no counts beyond its end): the read is issued early
+    // and its result taken where it is needed
+    auto lookup_issue = [&](int tau) -> int4 {
+      const int e = 2 * tau;
+      int4 v = make_int4(-1, 0, -1, 0);
+      if (e < n_union) v = *reinterpret_cast<const int4*>(walk + e);
+      return v;
     };
-    auto fetch_u = [&](int buf, int32_t ba, int32_t bb) {  // K and V rows of blocks A, B -> buffers buf (no B: block 0 again)
-      char* kb = buf ? k_buf[1] : k_buf[0];
-      char* vb = buf ? v_buf[1] : v_buf[0];
-#pragma unroll
-      for (int s = 0; s < 2; s++) {
-        const int32_t blk = s == 0 ? ba : bb;
-        const int64_t start = (int64_t)(blk < 0 ? 0 : blk) * 16;
-        const int last = (int)((N - start < 16 ? N - start : 16) - 1);
-        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + start * p.svn), 0, 0x7fffffff, 0x00020000);
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-          const int ldsrow = 16 * s + 8 * t + lr;
-          int row = 8 * t + lr;
-          row = row < last ? row : last;
-          const uint32_t kc = (uint32_t)(((lane & 7) ^ (ldsrow & 7)) * 16);
-          const uint32_t vc = (uint32_t)(((lane & 7) ^ (((ldsrow >> 1) & 1) << 2)) * 16);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(kb + (2 * s + t) * 1024), 16,
-                                                   (uint32_t)row * krow + kc, 0, 0, 0);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(vb + (2 * s + t) * 1024), 16,
-                                                   (uint32_t)row * vrow + vc, 0, 0, 0);
-        }
-      }
+    auto lookup_take = [&](const int4& v, int32_t& a, uint32_t& ca, int32_t& b2, uint32_t& cb) {
+      a = __builtin_amdgcn_readfirstlane(v.x);
+      ca = (uint32_t)__builtin_amdgcn_readfirstlane(v.y);
+      b2 = __builtin_amdgcn_readfirstlane(v.z);
+      cb = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
     };
-    V8 ak[4];       // K fragments of the current tile
-    V8 vfr[2][2];   // V^T fragments of the current tile [jj][dt]
-    auto load_frags = [&](int buf) {
-      const char* kb = buf ? k_buf[1] : k_buf[0];
-      const char* vb = buf ? v_buf[1] : v_buf[0];
+
+    // ---- transfers: one descriptor per tensor, the block's byte offset rides in the scalar offset ----
+    const uint32_t koff = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ lr) * 16);
+    const uint32_t voff = (uint32_t)lr * vrow + (uint32_t)(((lane & 7) ^ (((lr >> 1) & 1) << 2)) * 16);
+    typedef __attribute__((address_space(3))) char* LdsPtr;  // arithmetic stays in the LDS address space (no null checks)
+    const LdsPtr k_lds[2] = {(LdsPtr)lds_k0 + wave * kHalfBytes, (LdsPtr)lds_k1 + wave * kHalfBytes};
+    const LdsPtr v_lds[2] = {(LdsPtr)lds_v0 + wave * kHalfBytes, (LdsPtr)lds_v1 + wave * kHalfBytes};
+    // 16 rows of one block -> 2 KB at dst.  The instruction's immediate offset moves the LDS side and the global side
+    // alike; the scalar offset makes up the difference (row strides are at least 128 bytes).
+    auto dma_block = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t rowb, int32_t blk) {
+      const uint32_t so = (uint32_t)blk * 16u * rowb;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off0, so, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off0, so + (8u * rowb - 1024u), 1024, 0);
+    };
+    auto dma_ragged = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t rowb) {  // rows beyond the sequence re-read its last row
+      const uint32_t so = (uint32_t)ragged_blk * 16u * rowb;
+      const int r0 = lr < ragged_last ? lr : ragged_last, r1 = 8 + lr < ragged_last ? 8 + lr : ragged_last;
+      const uint32_t col = off0 - (uint32_t)lr * rowb;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (uint32_t)r0 * rowb + col, so, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst + 1024, 16, (uint32_t)r1 * rowb + col, so, 0, 0);
+    };
+    // A tile beyond the end of the list (a < 0) is requested all the same, through a descriptor of zero records:
+    // every lane is out of range, nothing is fetched, and the count of outstanding transfers does not depend on the
+    // list (the waits below are constants).  No second block: the first one again (finite scores).
+    auto records = [](int32_t a) -> int32_t {  // -1 (no limit) for a block, 0 for none; scalar instructions by hand: the
+      int32_t r;                               // compiler's own select lands in a vector register and the descriptor with it
+      asm("s_ashr_i32 %0, %1, 31\n\ts_not_b32 %0, %0" : "=s"(r) : "s"(a) : "scc");
+      return r;
+    };
+    auto dma_k = [&](auto par_tag, int32_t a, int32_t b2) {
+      constexpr int P = decltype(par_tag)::value;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, records(a), 0x00020000);
+      dma_block(rs, k_lds[P], koff, krow, a);
+      dma_block(rs, k_lds[P] + 2048, koff, krow, b2 < 0 ? a : b2);
+    };
+    auto dma_v = [&](auto par_tag, int32_t a, int32_t b2) {
+      constexpr int P = decltype(par_tag)::value;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, records(a), 0x00020000);
+      dma_block(rs, v_lds[P], voff, vrow, a);
+      dma_block(rs, v_lds[P] + 2048, voff, vrow, b2 < 0 ? a : b2);
+    };
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, -1, 0x00020000);
+    V8 ak[4];       // K fragments of one tile
+    V8 vfr[2][2];   // V^T fragments of one tile [jj][dt]
+    auto load_k = [&](auto par_tag) {
+      constexpr int P = decltype(par_tag)::value;
+      const char* kb = P ? k_buf[1] : k_buf[0];
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
         Frag f;
         f.u = *reinterpret_cast<const uint4*>(kb + (kr_off ^ (ks << 5)));
         ak[ks] = as_v8<E>(f);
       }
+    };
+    auto load_v = [&](auto par_tag) {
+      constexpr int P = decltype(par_tag)::value;
+      const char* vb = P ? v_buf[1] : v_buf[0];
 #pragma unroll
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
@@ -295,137 +359,190 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
           vfr[jj][dt] = as_v8<E>(f);
         }
     };
-    auto compute_u = [&](int32_t ba, uint32_t ca, int32_t bb, uint32_t cb) {  // on the fragments in registers
-      const int nka = (int)(N - (int64_t)ba * 16 < 16 ? N - (int64_t)ba * 16 : 16);
-      const int nkb = bb < 0 ? 0 : (int)(N - (int64_t)bb * 16 < 16 ? N - (int64_t)bb * 16 : 16);
-      const int mine = c >> 4;
-      // The three stages of a 32-query half (one half after the other: interleaving the two halves' stages was slower).
-      f32x16 st[2];
-      union { V8 v; } pf[2][2];
-      auto scores = [&](auto qt_tag) {
-        constexpr int QT = decltype(qt_tag)::value;
+
+    // ---- the arithmetic of a unit ----
+    f32x16 st[2];     // scores of the two halves (unit (t, 1) and unit (t, 0) or (t + 1, 0))
+    V8 pf[2][2];      // probabilities [half][jj: block A, B]
+    float nega[2], negb[2];  // what is added in the exponent for block A / B: minus the reference, or -inf if not listed
+    bool exact = false;      // second walk: running maximum
+    const int mine = c >> 4;  // the lane's query block within the half
+    // Register r of st[QT]: key row 4hh + 8((r%8)/4) + r%4 of block A (r < 8) or B (r >= 8).
+    // Softmax reference.  First walk (exact == false): a query's reference is the maximum over the first tile that
+    // holds a block of its list and then stays (softmax is shift invariant), so later tiles need no maximum, no
+    // comparison and no pass over the accumulators; probabilities may exceed 1, and a row sum that ends up huge or
+    // not finite sends the group through a second walk with the running maximum (exact == true).
+    auto pre = [&](auto qt_tag, uint32_t ca, uint32_t cb) {
+      constexpr int QT = decltype(qt_tag)::value;
+      const uint32_t pa = (ca >> (16 * QT)) & 0xffffu, pb = (cb >> (16 * QT)) & 0xffffu;  // the half's two query blocks
+      const int wa = (int)(mine ? pa >> 8 : pa & 0xffu), wb = (int)(mine ? pb >> 8 : pb & 0xffu);
+      const bool unset = m_i[QT] == -INFINITY && (wa | wb) != 0;
+      if (exact || __any(unset)) {
+        float mxa = st[QT][0], mxb = st[QT][8];
 #pragma unroll
-        for (int r = 0; r < 16; r++) st[QT][r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) st[QT] = Mma<E>::mma(ak[ks], bq[QT][ks], st[QT]);
-      };
-      auto softmax = [&](auto qt_tag) {
-        constexpr int QT = decltype(qt_tag)::value;
-        const uint32_t pa = (ca >> (16 * QT)) & 0xffffu, pb = (cb >> (16 * QT)) & 0xffffu;  // the half's two query blocks
-        const int wa = (int)(mine ? pa >> 8 : pa & 0xffu), wb = (int)(mine ? pb >> 8 : pb & 0xffu);
-        // register r: key row 4hh + 8((r%8)/4) + r%4 of block A (r < 8) or B (r >= 8).  A block that the lane's query
-        // block does not list is left out through two per-lane constants (its maximum is dropped and its exponent gets
-        // -inf added); only the ragged last block needs per-register masks.
-        if (__any((wa && nka < 16) || (wb && nkb < 16))) {
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            const int row = 4 * hh + 8 * (j >> 2) + (j & 3);
-            if (row >= nka) st[QT][j] = -INFINITY;
-            if (row >= nkb) st[QT][8 + j] = -INFINITY;
-          }
+        for (int r = 1; r < 8; r++) {
+          mxa = fmaxf(mxa, st[QT][r]);
+          mxb = fmaxf(mxb, st[QT][8 + r]);
         }
-        // Softmax reference.  First walk (exact == false): a query's reference is the maximum over the first tile that
-        // holds a block of its list and then stays (softmax is shift invariant), so later tiles need no maximum, no
-        // comparison and no pass over the accumulators; probabilities may exceed 1, and a row sum that ends up huge or
-        // not finite sends the group through a second walk with the running maximum (exact == true).
-        const bool unset = m_i[QT] == -INFINITY && (wa | wb) != 0;
-        if (exact || __any(unset)) {
-          float mxa = st[QT][0], mxb = st[QT][8];
+        float mx = fmaxf(wa ? mxa : -INFINITY, wb ? mxb : -INFINITY);
+        mx = xh_max(mx) * sl2;
+        const float m_new = (exact || unset) ? fmaxf(m_i[QT], mx) : m_i[QT];
+        if (__any(m_new != m_i[QT])) {
+          const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - (m_new == -INFINITY ? 0.f : m_new));  // 0 while m_i is -inf
+          l_i[QT] *= alpha;
 #pragma unroll
-          for (int r = 1; r < 8; r++) {
-            mxa = fmaxf(mxa, st[QT][r]);
-            mxb = fmaxf(mxb, st[QT][8 + r]);
-          }
-          float mx = fmaxf(wa ? mxa : -INFINITY, wb ? mxb : -INFINITY);
-          mx = xh_max(mx) * sl2;
-          const float m_new = (exact || unset) ? fmaxf(m_i[QT], mx) : m_i[QT];
-          if (__any(m_new != m_i[QT])) {
-            const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - (m_new == -INFINITY ? 0.f : m_new));  // 0 while m_i is -inf
-            l_i[QT] *= alpha;
+          for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-              for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
-          }
-          m_i[QT] = m_new;
+            for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
         }
-        const float m_use = m_i[QT] == -INFINITY ? 0.f : m_i[QT];
-        const float nega = wa ? -m_use : -INFINITY, negb = wb ? -m_use : -INFINITY;  // -inf: every probability 0
-        const bool dup = __any(wa > 1 || wb > 1);
-        const float fa = (float)wa, fb = (float)wb;
-#pragma unroll
-        for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            float x0 = __builtin_amdgcn_exp2f(fmaf(st[QT][8 * jj + e], sl2, jj == 0 ? nega : negb));
-            float x1 = __builtin_amdgcn_exp2f(fmaf(st[QT][8 * jj + e + 1], sl2, jj == 0 ? nega : negb));
-            if (dup) {  // a list that names the block more than once attends it that often
-              x0 *= jj == 0 ? fa : fb;
-              x1 *= jj == 0 ? fa : fb;
-            }
-            V2 pk;
-            pk[0] = (E)x0;
-            pk[1] = (E)x1;
-            pf[QT][jj].v[e] = pk[0];
-            pf[QT][jj].v[e + 1] = pk[1];
-            l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
-          }
-      };
-      auto values = [&](auto qt_tag) {
-        constexpr int QT = decltype(qt_tag)::value;
-#pragma unroll
-        for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-          for (int dt = 0; dt < 2; dt++) ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[QT][jj].v, ot[dt][QT]);
-      };
-      // (wave-uniform) does some query of the half list A or B?
-      const bool act0 = ((ca | cb) & 0xffffu) != 0, act1 = ((ca | cb) >> 16) != 0;
-      if (act0) {
-        scores(H0{});
-        softmax(H0{});
-        values(H0{});
+        m_i[QT] = m_new;
       }
-      if (act1) {
-        scores(H1{});
-        softmax(H1{});
-        values(H1{});
+      const float m_use = m_i[QT] == -INFINITY ? 0.f : m_i[QT];
+      if (dup) {  // a list that names the block w times attends it w times: w exp2(x) = exp2(x + log2 w), log2 0 = -inf
+        nega[QT] = __builtin_amdgcn_logf((float)wa) - m_use;
+        negb[QT] = __builtin_amdgcn_logf((float)wb) - m_use;
+      } else {
+        nega[QT] = wa ? -m_use : -INFINITY;
+        negb[QT] = wb ? -m_use : -INFINITY;
       }
     };
+    // two of the unit's 16 exponentials (slot J of 8).  Row sums over the ROUNDED probabilities: with a reference below
+    // the maximum a probability is not a power of two, and its rounding cancels in p / sum p only if the sum has it too
+    auto exps = [&](auto qt_tag, auto j_tag) {
+      constexpr int QT = decltype(qt_tag)::value;
+      constexpr int r = 2 * decltype(j_tag)::value, jj = r >> 3, e8 = r & 7;
+      asm volatile("" : "+v"(st[QT]));
+      const float ng = jj ? negb[QT] : nega[QT];
+      const float x0 = __builtin_amdgcn_exp2f(fmaf(st[QT][r], sl2, ng));
+      const float x1 = __builtin_amdgcn_exp2f(fmaf(st[QT][r + 1], sl2, ng));
+      V2 pk;
+      pk[0] = (E)x0;
+      pk[1] = (E)x1;
+      pf[QT][jj][e8] = pk[0];
+      pf[QT][jj][e8 + 1] = pk[1];
+      l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
+      asm volatile("" : "+v"(pf[QT][jj]), "+v"(l_i[QT]));
+    };
+    auto mma_s = [&](auto qt_tag, auto ks_tag) {  // scores of a half from the K fragments in registers
+      constexpr int QT = decltype(qt_tag)::value, ks = decltype(ks_tag)::value;
+      if constexpr (ks == 0) {
+        f32x16 z;
+#pragma unroll
+        for (int r = 0; r < 16; r++) z[r] = 0.f;
+        st[QT] = Mma<E>::mma(ak[0], bq[QT][0], z);
+      } else {
+        st[QT] = Mma<E>::mma(ak[ks], bq[QT][ks], st[QT]);
+      }
+    };
+    auto mma_pv = [&](auto qt_tag, auto i_tag) {  // O^T += V^T P^T of a half, V^T fragments in registers
+      constexpr int QT = decltype(qt_tag)::value, i = decltype(i_tag)::value, jj = i >> 1, dt = i & 1;
+      ot[dt][QT] = Mma<E>::mma(vfr[jj][dt], pf[QT][jj], ot[dt][QT]);
+    };
+    // Tile t, parity P.  On entry: st[0] = scores of unit (t, 0); ak = K(t); vfr = V(t-1); pf[1] = probabilities of
+    // unit (t-1, 1); in flight or landed: K(t+1), V(t) (older group), K(t+2), V(t+1) (newer group).
+    // ca, cb: the counts of the tile's blocks; (av, bv): tile t+2, whose V rows are requested here; nx: the pending
+    // read of tile t+3's entries, taken here into (a3, ca3, b3, cb3), whose K rows are requested here.
+    auto tile = [&](auto par_tag, uint32_t ca, uint32_t cb, int32_t av, int32_t bv, const int4& nx,
+                    int32_t& a3, uint32_t& ca3, int32_t& b3, uint32_t& cb3) {
+      constexpr int P = decltype(par_tag)::value;
+      typedef std::integral_constant<int, P ^ 1> Q;
+      pre(H0{}, ca, cb);
+      static_for<8>([&](auto j_tag) {  // exponentials of (t, 0); scores of (t, 1); PV of (t-1, 1)
+        constexpr int j = decltype(j_tag)::value;
+        if constexpr (j == 4) {
+          __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the older group has landed
+          load_k(Q{});                                   // K(t+1)
+        }
+        if constexpr (j < 4) mma_s(H1{}, j_tag);
+        else mma_pv(H1{}, std::integral_constant<int, j - 4>{});
+        exps(H0{}, j_tag);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      load_v(par_tag);  // V(t)
+      pre(H1{}, ca, cb);
+      static_for<8>([&](auto j_tag) {  // exponentials of (t, 1); scores of (t+1, 0); PV of (t, 0)
+        constexpr int j = decltype(j_tag)::value;
+        if constexpr (j == 2) {
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments of K(t+1) and V(t) are in registers
+          lookup_take(nx, a3, ca3, b3, cb3);
+          dma_k(Q{}, a3, b3);        // K(t+3) over K(t+1)
+          dma_v(par_tag, av, bv);    // V(t+2) over V(t)
+        }
+        if constexpr (j < 4) mma_s(H0{}, j_tag);
+        else mma_pv(H0{}, std::integral_constant<int, j - 4>{});
+        exps(H1{}, j_tag);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    };
+
+    const int ntiles = (n_union + 1) >> 1;
     for (int pass = 0; pass < 2; pass++) {
       exact = pass == 1;
-#pragma unroll
-      for (int j = 0; j < 4; j++) rem[j] = __ballot(my_idx[j] >= 0);
-      int32_t a0, b0;
-      uint32_t ca0, cb0;
-      pop(a0, ca0);
-      pop(b0, cb0);
-      if (a0 >= 0) {
-        int buf = 0;
+      if (ntiles > 0) {
+        int32_t a0, b0, a1, b1, a2, b2, a3, b3;  // blocks and counts of tiles t .. t+3
+        uint32_t ca0, cb0, ca1, cb1, ca2, cb2, ca3, cb3;
+        lookup_take(lookup_issue(0), a0, ca0, b0, cb0);
+        lookup_take(lookup_issue(1), a1, ca1, b1, cb1);
+        lookup_take(lookup_issue(2), a2, ca2, b2, cb2);
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): (second walk) the first walk's last reads are done
-        // Two tiles in flight: a tile's fragments go to registers in one go, which frees its buffers for the tile
-        // after the next before any arithmetic starts.
-        fetch_u(0, a0, b0);
-        int32_t a1, b1;
-        uint32_t ca1, cb1;
-        pop(a1, ca1);
-        pop(b1, cb1);
-        if (a1 >= 0) fetch_u(1, a1, b1);
-        while (true) {
-          if (a1 >= 0) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the current tile has landed (the next one may be in flight)
-          else __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
-          load_frags(buf);
-          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments are in registers, the buffers are free
-          int32_t a2, b2;
-          uint32_t ca2, cb2;
-          pop(a2, ca2);
-          pop(b2, cb2);
-          if (a2 >= 0) fetch_u(buf, a2, b2);
-          compute_u(a0, ca0, b0, cb0);
-          if (a1 < 0) break;
-          a0 = a1; ca0 = ca1; b0 = b1; cb0 = cb1;
-          a1 = a2; ca1 = ca2; b1 = b2; cb1 = cb2;
-          buf ^= 1;
+        dma_k(H0{}, a0, b0);
+        dma_k(H1{}, a1, b1);
+        dma_v(H0{}, a0, b0);
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): K(0) has landed
+        load_k(H0{});
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        dma_k(H0{}, a2, b2);
+        dma_v(H1{}, a1, b1);
+        static_for<4>([&](auto ks_tag) { mma_s(H0{}, ks_tag); });
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {  // nothing before unit (0, 0): its PV slot adds zero
+#pragma unroll
+          for (int e = 0; e < 8; e++) pf[1][jj][e] = (E)0.f;
+#pragma unroll
+          for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) vfr[jj][dt][e] = (E)0.f;
         }
+        int t = 0;
+        for (; t + 1 < ntiles; t += 2) {
+          int4 nx = lookup_issue(t + 3);
+          tile(H0{}, ca0, cb0, a2, b2, nx, a3, ca3, b3, cb3);
+          ca0 = ca1; cb0 = cb1;
+          ca1 = ca2; cb1 = cb2;
+          a2 = a3; b2 = b3; ca2 = ca3; cb2 = cb3;
+          nx = lookup_issue(t + 4);
+          tile(H1{}, ca0, cb0, a2, b2, nx, a3, ca3, b3, cb3);
+          ca0 = ca1; cb0 = cb1;
+          ca1 = ca2; cb1 = cb2;
+          a2 = a3; b2 = b3; ca2 = ca3; cb2 = cb3;
+        }
+        if (t < ntiles) {  // an odd number of tiles: the last one (nothing left to request)
+          const int4 none = make_int4(-1, 0, -1, 0);
+          tile(H0{}, ca0, cb0, -1, -1, none, a3, ca3, b3, cb3);
+        }
+        static_for<4>([&](auto i_tag) { mma_pv(H1{}, i_tag); });  // PV of the last unit
+      }
+      if (ragged_cnts != 0) {  // the block that ends the sequence early: one unpipelined step with the running maximum
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): earlier reads of the buffers are done
+        dma_ragged(rk, k_lds[0], koff, krow);
+        dma_ragged(rk, k_lds[0] + 2048, koff, krow);  // the tile's second block: the same rows again (finite values)
+        dma_ragged(rv, v_lds[0], voff, vrow);
+        dma_ragged(rv, v_lds[0] + 2048, voff, vrow);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        load_k(H0{});
+        load_v(H0{});
+        const bool was_exact = exact;
+        exact = true;
+        static_for<2>([&](auto qt_tag) {
+          constexpr int QT = decltype(qt_tag)::value;
+          static_for<4>([&](auto ks_tag) { mma_s(qt_tag, ks_tag); });
+#pragma unroll
+          for (int j = 0; j < 8; j++)
+            if (4 * hh + 8 * (j >> 2) + (j & 3) > ragged_last) st[QT][j] = -INFINITY;
+          pre(qt_tag, ragged_cnts, 0u);
+          static_for<8>([&](auto j_tag) { exps(qt_tag, j_tag); });
+          static_for<4>([&](auto i_tag) { mma_pv(qt_tag, i_tag); });
+        });
+        exact = was_exact;
       }
       const float big = 1.2676506e30f;  // 2^100
       if (exact || !__any(!(l_i[0] < big) || !(l_i[1] < big))) break;
@@ -530,10 +647,14 @@ int launch_select_b16(const AttnParams& p, int dtype, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)total), blk(64 * b16::kWaves);
   // default: the union walk; S3R_B16_KERNEL=pairs picks the walk over pairs of list entries (kept as a cross-check)
-  static const bool pairs = [] {
+  static const bool pairs_env = [] {
     const char* e = getenv("S3R_B16_KERNEL");
     return e != nullptr && strcmp(e, "pairs") == 0;
   }();
+  // the union walk addresses a head's K and V rows through 32-bit byte offsets from one descriptor per tensor
+  const int64_t es = 2;
+  const bool wide = (p.Lq - 1) * p.skn * es + 128 > 0xffffffffLL || (p.Lq - 1) * p.svn * es + 128 > 0xffffffffLL;
+  const bool pairs = pairs_env || wide;
 #define S3R_B16(E, U) hipLaunchKernelGGL((b16::select_b16_kernel<E, U>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total)
   if (dtype == S3R_BF16) {
     if (pairs) S3R_B16(bf16_t, false); else S3R_B16(bf16_t, true);
