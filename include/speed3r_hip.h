@@ -83,6 +83,29 @@ int s3r_compressed_attn_topk(const void* q, const void* k, const void* v,
                              float softmax_scale, int dtype, void* stream);
 
 /*
+ * The causal variant of s3r_compressed_attn_topk: the IS_CAUSAL branches of _fwd_kernel_with_topk
+ * (flash_attention_topk.py:71,93), which the reference layer never takes (it calls with causal=False).
+ * Query i (row i of its 64-row block m = i / 64) sees the keys below end_n = min((m + 1) * 64, Lk) only:
+ *   o, lse:   softmax over the keys j <= i;
+ *   topk_idx: the K largest of the keys j < end_n, where a key j > i has the score -inf (it ranks below every finite
+ *             score, lowest column first, as the reference's integer keys order it); if end_n < K the trailing slots
+ *             hold end_n - 1;
+ *   scores:   [B,H,Lq,Lk] fp32 work buffer, required with `topk_idx` (row i: raw scores of the keys j < end_n with
+ *             -inf for j > i; columns from end_n on are not written).
+ * Any I/O dtype, D <= 64, K a power of two <= 64; runs the generic (non-MFMA) kernels.  The reference's backward
+ * ignores `causal` (flash_attention_topk.py:653-666 calls _flash_attn_backward without it), so s3r_attn_bwd on the
+ * lse of this call reproduces the reference's gradients as they are.
+ */
+int s3r_compressed_attn_topk_causal(const void* q, const void* k, const void* v,
+                                    void* o, float* lse, int32_t* topk_idx, float* scores,
+                                    int B, int H, int Lq, int Lk, int D, int K,
+                                    int64_t sqb, int64_t sqh, int64_t sqm,
+                                    int64_t skb, int64_t skh, int64_t skn,
+                                    int64_t svb, int64_t svh, int64_t svn,
+                                    int64_t sob, int64_t soh, int64_t som,
+                                    float softmax_scale, int dtype, void* stream);
+
+/*
  * s3r_compressed_attn_topk with its score buffer built into the library: allocates nothing.
  * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It is the `scores != NULL` path of

@@ -25,6 +25,9 @@ SIGNATURES = {
     "s3r_compressed_attn_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_int, c_int, c_int, c_int, c_int, c_int,
                                          *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
+    "s3r_compressed_attn_topk_causal": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int, c_int, c_int, c_int, c_int, c_int,
+                                         *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),
     "s3r_compressed_attn_topk_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                 c_int, c_int, c_int, c_int, c_int, c_int,
                                                 *_i64x3, *_i64x3, *_i64x3, *_i64x3, c_float, c_int, c_void_p]),

@@ -64,6 +64,31 @@ extern "C" int s3r_compressed_attn_topk(const void* q, const void* k, const void
   return rc;
 }
 
+extern "C" int s3r_compressed_attn_topk_causal(const void* q, const void* k, const void* v, void* o, float* lse, int32_t* topk_idx,
+                                               float* scores, int B, int H, int Lq, int Lk, int D, int K,
+                                               int64_t sqb, int64_t sqh, int64_t sqm, int64_t skb, int64_t skh, int64_t skn,
+                                               int64_t svb, int64_t svh, int64_t svn, int64_t sob, int64_t soh, int64_t som,
+                                               float softmax_scale, int dtype, void* stream) {
+  if (!q || !k || !v || !o) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk_causal: null pointer");
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || D <= 0) return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk_causal: non-positive size");
+  if (!dtype_ok(dtype)) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk_causal: dtype %d", dtype);
+  if (D > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk_causal: head_dim %d > 64", D);
+  if (topk_idx != nullptr && (K < 1 || K > 64 || (K & (K - 1)) != 0))
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk_causal: top-k %d must be a power of two <= 64", K);
+  if (topk_idx != nullptr && scores == nullptr)
+    return fail(S3R_ERR_BAD_ARG, "s3r_compressed_attn_topk_causal: the indices are selected from a score buffer; pass one");
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.scores = scores; p.idx = nullptr; p.topk_idx = topk_idx;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk; p.D = D; p.block = 64; p.K = K; p.causal = 1;
+  p.sqb = sqb; p.sqh = sqh; p.sqm = sqm; p.skb = skb; p.skh = skh; p.skn = skn;
+  p.svb = svb; p.svh = svh; p.svn = svn; p.sob = sob; p.soh = soh; p.som = som;
+  p.scale = softmax_scale;
+  int rc = launch_attn_simple(p, dtype, /*select=*/false, stream);
+  if (rc != S3R_OK) return rc;
+  if (topk_idx != nullptr) rc = launch_topk_rows(scores, topk_idx, (int64_t)B * H * Lq, Lk, Lk, K, Lq, stream);
+  return rc;
+}
+
 // ---- the entry point that allocates nothing --------------------------------------------------
 // Score buffer of s3r_compressed_attn_topk_static: device memory owned by the code object, one copy per GPU at
 // its own address, held until the process ends.  The name below is only a handle for hipGetSymbolAddress; host

@@ -16,6 +16,7 @@ struct AttnParams {
   int B, H;
   int64_t Lq, Lk;
   int D, block, K;
+  int causal;          // compressed branch, generic kernel: key j counts for query i only if j <= i, see attn_simple.hip
   int64_t sqb, sqh, sqm;
   int64_t skb, skh, skn;
   int64_t svb, svh, svn;
@@ -32,6 +33,8 @@ struct AttnParams {
 };
 
 // launchers implemented in the .hip files; each returns S3R_OK or an error code
+// row-wise top-k; causal_lq > 0: row r (query r % causal_lq) ranks only its first min((q/64 + 1) * 64, cols) columns
+int launch_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int64_t row_stride, int K, int64_t causal_lq, void* stream);
 int launch_attn_simple(const AttnParams& p, int dtype, bool select, void* stream);
 int launch_select_pipe(const AttnParams& p, int dtype, void* stream);
 int launch_select_b16(const AttnParams& p, int dtype, void* stream);  // block 16

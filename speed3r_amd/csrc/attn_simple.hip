@@ -8,6 +8,10 @@
 // registers; K, V and the probability tile go through LDS as fp32.  All arithmetic is fp32
 // FMA; probabilities are rounded to the I/O dtype before the PV product as the reference's
 // kernels do (a no-op for fp32 I/O).
+//
+// Causal variant of the compressed branch (p.causal; flash_attention_topk.py:71,93): a 64-row query block walks the
+// key tiles below end_n = min((block + 1) * 64, Lk) only, and key j > query i gets the score -inf, in the softmax
+// and in the stored score (the reference ranks such keys, below every finite score, lowest column first).
 #include "s3r_common.h"
 #include "attn_params.h"
 
@@ -45,7 +49,9 @@ __global__ __launch_bounds__(256) void attn_simple_kernel(AttnParams p) {
 #pragma unroll
   for (int i = 0; i < 16; i++) acc[i] = 0.f;
 
-  const int ntiles = SELECT ? p.K : (int)((p.Lk + 63) / 64);
+  const bool causal = !SELECT && p.causal != 0;
+  const int64_t end_n = causal ? ((mblk + 1) * 64 < p.Lk ? (mblk + 1) * 64 : p.Lk) : p.Lk;
+  const int ntiles = SELECT ? p.K : (int)((end_n + 63) / 64);
   const int32_t* idx_row = SELECT ? p.idx + (int64_t)b * p.sib + (int64_t)h * p.sih + mblk * p.sim : nullptr;
 
   for (int t = 0; t < ntiles; t++) {
@@ -84,7 +90,7 @@ __global__ __launch_bounds__(256) void attn_simple_kernel(AttnParams p) {
         a = fmaf(qreg[4 * d4 + 2], kv.z, a);
         a = fmaf(qreg[4 * d4 + 3], kv.w, a);
       }
-      s[i] = a;
+      s[i] = (causal && start + c > qrow) ? -INFINITY : a;
     }
     if (!SELECT && p.scores != nullptr && qvalid) {
       float* srow = p.scores + (((int64_t)b * p.H + h) * p.Lq + qrow) * p.Lk + start;
@@ -99,7 +105,7 @@ __global__ __launch_bounds__(256) void attn_simple_kernel(AttnParams p) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int c = g + 4 * i;
-      s[i] = (c < nvalid) ? s[i] * p.scale : -INFINITY;
+      s[i] = (c < nvalid && s[i] != -INFINITY) ? s[i] * p.scale : -INFINITY;  // (-inf * a non-positive scale)
       mx = fmaxf(mx, s[i]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 1));
@@ -110,7 +116,7 @@ __global__ __launch_bounds__(256) void attn_simple_kernel(AttnParams p) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int c = g + 4 * i;
-      const float pv = (c < nvalid) ? expf(s[i] - m_new) : 0.f;
+      const float pv = (c < nvalid && s[i] != -INFINITY) ? expf(s[i] - m_new) : 0.f;
       rowsum += pv;
       Ps[r * kLd + c] = round_to<T>(pv);
     }

@@ -57,10 +57,16 @@ struct RowTopK {
 };
 
 __global__ __launch_bounds__(256) void topk_rows_kernel(const float* __restrict__ scores, int32_t* __restrict__ idx,
-                                                        int64_t rows, int cols, int64_t row_stride, int K, int vec_ok) {
+                                                        int64_t rows, int cols_all, int64_t row_stride, int K, int vec_ok,
+                                                        int64_t causal_lq) {
   const int lane = threadIdx.x & 63;
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (w >= rows) return;
+  int cols = cols_all;
+  if (causal_lq > 0) {  // the causal kernel's 64-row query block stops at end_n (flash_attention_topk.py:71)
+    const int64_t end_n = ((w % causal_lq) / 64 + 1) * 64;
+    if (end_n < cols) cols = (int)end_n;
+  }
   const float* row = scores + w * row_stride;
   RowTopK st;
   st.init(K, lane);
@@ -134,8 +140,9 @@ __global__ __launch_bounds__(256) void topk_rows_kernel(const float* __restrict_
 
 using namespace s3r;
 
-extern "C" int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int64_t row_stride, int K,
-                             void* stream) {
+namespace s3r {
+int launch_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int64_t row_stride, int K, int64_t causal_lq,
+                     void* stream) {
   if (!scores || !idx) return fail(S3R_ERR_BAD_ARG, "s3r_topk_rows: null pointer");
   if (rows <= 0 || cols <= 0 || row_stride < cols) return fail(S3R_ERR_BAD_ARG, "s3r_topk_rows: bad rows/cols/stride");
   if (K < 1 || K > 64) return fail(S3R_ERR_UNSUPPORTED, "s3r_topk_rows: K=%d outside [1,64]", K);
@@ -143,6 +150,12 @@ extern "C" int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, in
   if (nwg > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_topk_rows: too many rows");
   const int vec_ok = aligned16(scores) && (row_stride % 4 == 0);
   hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)nwg), dim3(256), 0, (hipStream_t)stream, scores, idx, rows, cols,
-                     row_stride, K, vec_ok);
+                     row_stride, K, vec_ok, causal_lq);
   return check_launch("s3r_topk_rows");
+}
+}  // namespace s3r
+
+extern "C" int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int64_t row_stride, int K,
+                             void* stream) {
+  return launch_topk_rows(scores, idx, rows, cols, row_stride, K, 0, stream);
 }

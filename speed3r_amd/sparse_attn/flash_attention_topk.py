@@ -19,16 +19,18 @@ def flash_attn_topk_func(q, k, v, topk_val, bias=None, causal=False, softmax_sca
     Returns ``(o, topk_indices)``: ``o`` has q's shape and dtype; ``topk_indices`` is int32
     ``[batch, nheads, seqlen_q, topk_val]`` holding, for every query row, the columns of the
     ``topk_val`` largest raw (unscaled) fp32 scores in descending order, equal scores lowest
-    column first.  ``bias`` is unused by the reference kernel and must be None; the causal
-    variant is never taken by the reference layer and is not provided.
+    column first.
+
+    ``bias`` is accepted and ignored, as in the reference (``FlashAttnTopkFunc.forward`` never hands it to
+    ``forward_with_topk``, flash_attention_topk.py:646-648).  ``causal=True`` is the kernel's IS_CAUSAL variant
+    (:71,93; the reference layer never asks for it): query i attends the keys j <= i and ranks the keys of the
+    tiles its 64-row block visits, ``j < min((i // 64 + 1) * 64, seqlen_k)``, those above i with the score -inf.
+    Its gradients are, as in the reference (:653-666), those of the non-causal operator on the causal
+    log-sum-exp.
     """
     headdim = q.shape[-1]
     assert topk_val <= _BLOCK_N, f"Top-K value ({topk_val}) cannot exceed BLOCK_N ({_BLOCK_N})"
     assert headdim <= _BLOCK_HEADDIM, "headdim must be less than or equal to BLOCK_HEADDIM"
     assert topk_val >= 1 and (topk_val & (topk_val - 1)) == 0, "Top-K value must be a power of two"
-    if bias is not None:
-        raise NotImplementedError("flash_attn_topk_func: bias is not supported (the reference kernel ignores it)")
-    if causal:
-        raise NotImplementedError("flash_attn_topk_func: the causal variant is not provided")
-    o, idx = ops.compressed_attn_topk_autograd(q, k, v, topk_val, softmax_scale)
+    o, idx = ops.compressed_attn_topk_autograd(q, k, v, topk_val, softmax_scale, causal=bool(causal))
     return o, idx

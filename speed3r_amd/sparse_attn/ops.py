@@ -81,12 +81,13 @@ def pool_qkv_packed(qkv: torch.Tensor, num_heads: int, block: int) -> Tuple[torc
 
 # largest fp32 score buffer compressed_attn_topk allocates for its own use (a caller that asks for the scores gets them whole)
 SCORE_BUFFER_BYTES = 1 << 30
+CAUSAL_SCORE_BYTES = 8 << 30   # the causal variant's score buffer is not banded
 
 
 def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Tensor], topk: Optional[int],
                          softmax_scale: Optional[float] = None, return_scores: bool = False,
                          return_lse: bool = False, materialize_scores: Optional[bool] = None,
-                         out: Optional[torch.Tensor] = None):
+                         out: Optional[torch.Tensor] = None, causal: bool = False):
     """Dense attention over pooled tokens plus, if ``topk`` is given, the top-k columns of the
     raw scores per query row.
 
@@ -102,7 +103,45 @@ def compressed_attn_topk(q: torch.Tensor, k: torch.Tensor, v: Optional[torch.Ten
 
     ``out``: a ``[B,H,Lq,D]`` tensor (or view, any strides on the first three dimensions, e.g. the
     ``permute(0, 2, 1, 3)`` of a ``[B,Lq,H,D]`` buffer) that receives the attention output instead of a fresh one.
+
+    ``causal``: the reference kernel's IS_CAUSAL variant (flash_attention_topk.py:71,93), never taken by the reference
+    layer: query i attends the keys j <= i and ranks the keys below ``min((i // 64 + 1) * 64, Lk)``, those above i
+    with the score -inf.  Generic kernels with a full ``[B,H,Lq,Lk]`` fp32 score buffer (at most
+    ``CAUSAL_SCORE_BYTES``); with ``return_scores`` the columns a row does not rank are returned as NaN.
     """
+    if causal:
+        assert v is not None and out is None, "causal: attention output and indices come from one call, into a fresh tensor"
+        _need_device(q, k, v)
+        _forward_only(q, k, v)
+        q, k, v = (_last_contig(t) for t in (q, k, v))
+        assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
+        b, h, lq, d = q.shape
+        lk = k.shape[2]
+        assert k.shape == (b, h, lk, d) and v.shape == (b, h, lk, d), "k/v shape mismatch"
+        scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+        o = torch.empty_like(q, memory_format=torch.contiguous_format)
+        idx = torch.empty((b, h, lq, topk), dtype=torch.int32, device=q.device) if topk else None
+        lse = torch.empty((b, h, lq), dtype=torch.float32, device=q.device) if return_lse else None
+        scores = None
+        if topk or return_scores:
+            if 4 * b * h * lq * lk > CAUSAL_SCORE_BYTES:
+                raise RuntimeError(f"causal top-k keeps all {b}x{h}x{lq}x{lk} fp32 scores in one buffer; that exceeds "
+                                   f"CAUSAL_SCORE_BYTES = {CAUSAL_SCORE_BYTES}")
+            scores = torch.full((b, h, lq, lk), float("nan"), dtype=torch.float32, device=q.device) if return_scores \
+                else torch.empty((b, h, lq, lk), dtype=torch.float32, device=q.device)
+        st3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+        with torch.cuda.device(q.device):
+            rc = _lib.lib().s3r_compressed_attn_topk_causal(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if lse is not None else None,
+                idx.data_ptr() if idx is not None else None, scores.data_ptr() if scores is not None else None,
+                b, h, lq, lk, d, topk or 0, *st3(q), *st3(k), *st3(v), *st3(o), scale, _code(q), _stream(q))
+        _lib.check(rc, "s3r_compressed_attn_topk_causal")
+        res = [o, idx]
+        if return_scores:
+            res.append(scores)
+        if return_lse:
+            res.append(lse)
+        return tuple(res)
     indices_only = v is None
     if indices_only:
         assert topk and not return_scores and not return_lse and materialize_scores is not True, \
@@ -511,9 +550,9 @@ class _CompressedAttnFn(torch.autograd.Function):
     FlashAttnTopkFunc, flash_attention_topk.py:633-665)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, topk, softmax_scale):
+    def forward(ctx, q, k, v, topk, softmax_scale, causal=False):
         with torch.no_grad():
-            o, idx, lse = compressed_attn_topk(q, k, v, topk, softmax_scale, return_lse=True)
+            o, idx, lse = compressed_attn_topk(q, k, v, topk, softmax_scale, return_lse=True, causal=causal)
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.scale = softmax_scale
         if idx is not None:
@@ -525,7 +564,7 @@ class _CompressedAttnFn(torch.autograd.Function):
         q, k, v, o, lse = ctx.saved_tensors
         dq, dk, dv = attn_bwd(q, k, v, o, dout, lse, None, 64, ctx.scale,
                               need_dq=ctx.needs_input_grad[0], need_dkv=ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
-        return dq, dk, dv, None, None
+        return dq, dk, dv, None, None, None   # (the reference's backward does not know of `causal` either, :653-666)
 
 
 def _wants_grad(*ts: torch.Tensor) -> bool:
@@ -544,13 +583,13 @@ def select_attn_autograd(q, k, v, idx, block, softmax_scale=None):
     return _SelectAttnFn.apply(q, k, v, idx, block, softmax_scale)
 
 
-def compressed_attn_topk_autograd(q, k, v, topk, softmax_scale=None):
+def compressed_attn_topk_autograd(q, k, v, topk, softmax_scale=None, causal=False):
     """:func:`compressed_attn_topk` (``(o, idx)``), differentiable in q, k, v where the backward kernels are built."""
     if not _wants_grad(q, k, v):
-        return compressed_attn_topk(q, k, v, topk, softmax_scale)
+        return compressed_attn_topk(q, k, v, topk, softmax_scale, causal=causal)
     if not bwd_supported(q):
         raise RuntimeError("speed3r_amd: the attention backward is built for bf16/fp16, head_dim 64 only")
-    return _CompressedAttnFn.apply(q, k, v, topk, softmax_scale)
+    return _CompressedAttnFn.apply(q, k, v, topk, softmax_scale, causal)
 
 
 _SIDE_STREAMS = {}

@@ -184,8 +184,54 @@ def test_flash_attn_topk_func_signature():
     assert o.shape == q.shape and o.dtype == q.dtype
     assert idx.shape == (1, 2, 200, 16) and idx.dtype == torch.int32
     assert (idx[..., 0].cpu() == torch.arange(200)).float().mean() > 0.95     # q.q is (almost always) the row maximum
-    with pytest.raises(NotImplementedError):
-        s3r.flash_attn_topk_func(q.to(DEV), q.to(DEV), q.to(DEV), 16, None, True)
+    # bias is accepted and ignored, as in the reference (flash_attention_topk.py:646-648)
+    o2, idx2 = s3r.flash_attn_topk_func(q.to(DEV), q.to(DEV), q.to(DEV), 16, torch.ones((1, 2, 200, 200), device=DEV))
+    assert torch.equal(o2, o) and torch.equal(idx2, idx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lq,lk,k", [(150, 150, 16), (200, 200, 64), (100, 180, 8), (130, 70, 32), (40, 40, 64), (3, 2, 4), (1041, 1041, 16)])
+def test_causal_variant_matches_oracle(dtype, lq, lk, k):
+    """flash_attn_topk_func(causal=True), the reference kernel's IS_CAUSAL branches: attention within the dtype's
+    tolerance (1e-5 fp32, 2e-2 bf16/fp16), indices bit for bit from the scores the kernel stored, and those scores
+    against the oracle's (fp32 products in another order: 1e-4 of the largest score)."""
+    h = 2
+    q = _randn((1, h, lq, 64), 21, dtype, 0.5)
+    kk = _randn((1, h, lk, 64), 22, dtype, 0.5)
+    v = _randn((1, h, lk, 64), 23, dtype, 1.0)
+    o, idx, scores, lse = s3r.compressed_attn_topk(q.to(DEV), kk.to(DEV), v.to(DEV), k, causal=True, return_scores=True, return_lse=True)
+    want_o, want_lse, want_s = oracle.compressed_attention(q, kk, v, p_dtype=None if dtype == torch.float32 else dtype,
+                                                           out_dtype=torch.float32, causal=True)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert max_abs(o, want_o) <= tol
+    assert (lse.cpu() - want_lse).abs().max().item() <= 1e-4
+    sc = scores.cpu()
+    for m0 in range(0, lq, 64):
+        end_n = min(m0 + 64, lk)
+        got, want = sc[:, :, m0:m0 + 64, :end_n], want_s[:, :, m0:m0 + 64, :end_n]
+        assert torch.equal(torch.isinf(got), torch.isinf(want))
+        fin = torch.isfinite(want)
+        assert (got[fin] - want[fin]).abs().max().item() <= 1e-4 * max(1.0, want[fin].abs().max().item())
+        assert torch.isnan(sc[:, :, m0:m0 + 64, end_n:]).all()          # columns the block does not visit stay untouched
+    from oracle import sparse_attention_oracle as so
+    np.testing.assert_array_equal(idx.cpu().numpy(), so.topk_from_scores_causal(sc, k))
+    o2, idx2 = s3r.flash_attn_topk_func(q.to(DEV), kk.to(DEV), v.to(DEV), k, None, True)
+    assert torch.equal(o2, o) and torch.equal(idx2, idx)
+
+
+def test_causal_variant_backward_is_the_non_causal_backward_on_the_causal_lse():
+    """The reference's backward does not know of `causal` (flash_attention_topk.py:653-666): dq, dk, dv are those of
+    the dense operator evaluated with the forward's (causal) log-sum-exp and output."""
+    from speed3r_amd.sparse_attn import ops
+    lq = 200
+    q, kk, v = (_randn((1, 2, lq, 64), s, torch.bfloat16, 0.5).to(DEV).requires_grad_(True) for s in (31, 32, 33))
+    o, _ = s3r.flash_attn_topk_func(q, kk, v, 8, None, True)
+    g = _randn((1, 2, lq, 64), 34, torch.bfloat16, 1.0).to(DEV)
+    o.backward(g)
+    with torch.no_grad():
+        o_c, _, lse_c = ops.compressed_attn_topk(q, kk, v, 8, causal=True, return_lse=True)
+        dq, dk, dv = ops.attn_bwd(q, kk, v, o_c, g, lse_c, None, 64, None)
+    assert torch.equal(q.grad, dq) and torch.equal(kk.grad, dk) and torch.equal(v.grad, dv)
 
 
 # ------------------------------------------------------------------------------------ selection branch
