@@ -241,6 +241,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     //    unit u - 1, one MFMA per two exponentials.  K and V tiles come by direct transfers into two half buffers
     //    each, 1.5 tile times ahead of their use; all buffer choices are static (the loop is written for even and odd
     //    tiles), so that the only waits for transfers are the explicit ones.
+    uint64_t lanes_any[2];  // lanes (queries) of each half whose query block has at least one valid entry
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+      lanes_any[qt] = (__ballot(my_idx[2 * qt] >= 0) ? 0x0000FFFF0000FFFFull : 0ull) | (__ballot(my_idx[2 * qt + 1] >= 0) ? 0xFFFF0000FFFF0000ull : 0ull);
     __shared__ __attribute__((aligned(16))) int2 lds_walk[kWaves][264];  // up to 4 x 64 entries and the end mark
     int2* const walk = lds_walk[wave];
     const int32_t ragged_blk = (N & 15) ? (int32_t)(N >> 4) : -2;  // the block that ends before its 16th row ...
@@ -364,6 +368,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     f32x16 st[2];     // scores of the two halves (unit (t, 1) and unit (t, 0) or (t + 1, 0))
     V8 pf[2][2];      // probabilities [half][jj: block A, B]
     float nega[2], negb[2];  // what is added in the exponent for block A / B: minus the reference, or -inf if not listed
+    float negm[2] = {0.f, 0.f};  // minus the reference (0 while there is none)
+    bool settled[2];             // (wave-uniform) every query of the half that has a list has its reference
     bool exact = false;      // second walk: running maximum
     const int mine = c >> 4;  // the lane's query block within the half
     // Register r of st[QT]: key row 4hh + 8((r%8)/4) + r%4 of block A (r < 8) or B (r >= 8).
@@ -375,53 +381,68 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       constexpr int QT = decltype(qt_tag)::value;
       const uint32_t pa = (ca >> (16 * QT)) & 0xffffu, pb = (cb >> (16 * QT)) & 0xffffu;  // the half's two query blocks
       const int wa = (int)(mine ? pa >> 8 : pa & 0xffu), wb = (int)(mine ? pb >> 8 : pb & 0xffu);
-      const bool unset = m_i[QT] == -INFINITY && (wa | wb) != 0;
-      if (exact || __any(unset)) {
-        float mxa = st[QT][0], mxb = st[QT][8];
+      if (exact || !settled[QT]) {  // (wave-uniform) once every query with a list has its reference, none of this runs
+        const bool unset = m_i[QT] == -INFINITY && (wa | wb) != 0;
+        if (exact || __any(unset)) {
+          float mxa = st[QT][0], mxb = st[QT][8];
 #pragma unroll
-        for (int r = 1; r < 8; r++) {
-          mxa = fmaxf(mxa, st[QT][r]);
-          mxb = fmaxf(mxb, st[QT][8 + r]);
+          for (int r = 1; r < 8; r++) {
+            mxa = fmaxf(mxa, st[QT][r]);
+            mxb = fmaxf(mxb, st[QT][8 + r]);
+          }
+          float mx = fmaxf(wa ? mxa : -INFINITY, wb ? mxb : -INFINITY);
+          mx = xh_max(mx) * sl2;
+          const float m_new = (exact || unset) ? fmaxf(m_i[QT], mx) : m_i[QT];
+          if (__any(m_new != m_i[QT])) {
+            const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - (m_new == -INFINITY ? 0.f : m_new));  // 0 while m_i is -inf
+            l_i[QT] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
+          }
+          m_i[QT] = m_new;
+          negm[QT] = m_new == -INFINITY ? 0.f : -m_new;
         }
-        float mx = fmaxf(wa ? mxa : -INFINITY, wb ? mxb : -INFINITY);
-        mx = xh_max(mx) * sl2;
-        const float m_new = (exact || unset) ? fmaxf(m_i[QT], mx) : m_i[QT];
-        if (__any(m_new != m_i[QT])) {
-          const float alpha = __builtin_amdgcn_exp2f(m_i[QT] - (m_new == -INFINITY ? 0.f : m_new));  // 0 while m_i is -inf
-          l_i[QT] *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) ot[dt][QT][r] *= alpha;
-        }
-        m_i[QT] = m_new;
+        settled[QT] = (__ballot(m_i[QT] != -INFINITY) & lanes_any[QT]) == lanes_any[QT];
       }
-      const float m_use = m_i[QT] == -INFINITY ? 0.f : m_i[QT];
       if (dup) {  // a list that names the block w times attends it w times: w exp2(x) = exp2(x + log2 w), log2 0 = -inf
-        nega[QT] = __builtin_amdgcn_logf((float)wa) - m_use;
-        negb[QT] = __builtin_amdgcn_logf((float)wb) - m_use;
+        nega[QT] = __builtin_amdgcn_logf((float)wa) + negm[QT];
+        negb[QT] = __builtin_amdgcn_logf((float)wb) + negm[QT];
       } else {
-        nega[QT] = wa ? -m_use : -INFINITY;
-        negb[QT] = wb ? -m_use : -INFINITY;
+        nega[QT] = wa ? negm[QT] : -INFINITY;
+        negb[QT] = wb ? negm[QT] : -INFINITY;
       }
     };
-    // two of the unit's 16 exponentials (slot J of 8).  Row sums over the ROUNDED probabilities: with a reference below
-    // the maximum a probability is not a power of two, and its rounding cancels in p / sum p only if the sum has it too
-    auto exps = [&](auto qt_tag, auto j_tag) {
+    // Two of the unit's 16 exponentials per slot (8 slots).  A slot computes its pair and rounds / sums the pair of the
+    // slot before, so that no instruction waits on an exponential just issued.  Row sums over the ROUNDED
+    // probabilities: with a reference below the maximum a probability is not a power of two, and its rounding cancels
+    // in p / sum p only if the sum has it too.
+    float px0 = 0.f, px1 = 0.f;  // the pair in flight
+    auto exps_finish = [&](auto qt_tag, auto j_tag) {
       constexpr int QT = decltype(qt_tag)::value;
       constexpr int r = 2 * decltype(j_tag)::value, jj = r >> 3, e8 = r & 7;
-      asm volatile("" : "+v"(st[QT]));
-      const float ng = jj ? negb[QT] : nega[QT];
-      const float x0 = __builtin_amdgcn_exp2f(fmaf(st[QT][r], sl2, ng));
-      const float x1 = __builtin_amdgcn_exp2f(fmaf(st[QT][r + 1], sl2, ng));
       V2 pk;
-      pk[0] = (E)x0;
-      pk[1] = (E)x1;
+      pk[0] = (E)px0;
+      pk[1] = (E)px1;
       pf[QT][jj][e8] = pk[0];
       pf[QT][jj][e8 + 1] = pk[1];
       l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
-      asm volatile("" : "+v"(pf[QT][jj]), "+v"(l_i[QT]));
     };
+    auto exps = [&](auto qt_tag, auto j_tag) {
+      constexpr int QT = decltype(qt_tag)::value;
+      constexpr int j = decltype(j_tag)::value, r = 2 * j, jj = r >> 3;
+      asm volatile("" : "+v"(st[QT]));
+      if constexpr (j > 0) exps_finish(qt_tag, std::integral_constant<int, j - 1>{});
+      const float ng = jj ? negb[QT] : nega[QT];
+      px0 = __builtin_amdgcn_exp2f(fmaf(st[QT][r], sl2, ng));
+      px1 = __builtin_amdgcn_exp2f(fmaf(st[QT][r + 1], sl2, ng));
+      V8& pa = pf[QT][0];
+      V8& pb = pf[QT][1];
+      float& li = l_i[QT];
+      asm volatile("" : "+v"(pa), "+v"(pb), "+v"(li), "+v"(px0), "+v"(px1));
+    };
+    auto exps_tail = [&](auto qt_tag) { exps_finish(qt_tag, std::integral_constant<int, 7>{}); };
     auto mma_s = [&](auto qt_tag, auto ks_tag) {  // scores of a half from the K fragments in registers
       constexpr int QT = decltype(qt_tag)::value, ks = decltype(ks_tag)::value;
       if constexpr (ks == 0) {
@@ -457,6 +478,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
         exps(H0{}, j_tag);
         __builtin_amdgcn_sched_barrier(0);
       });
+      exps_tail(H0{});
       load_v(par_tag);  // V(t)
       pre(H1{}, ca, cb);
       static_for<8>([&](auto j_tag) {  // exponentials of (t, 1); scores of (t+1, 0); PV of (t, 0)
@@ -472,11 +494,14 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
         exps(H1{}, j_tag);
         __builtin_amdgcn_sched_barrier(0);
       });
+      exps_tail(H1{});
     };
 
     const int ntiles = (n_union + 1) >> 1;
     for (int pass = 0; pass < 2; pass++) {
       exact = pass == 1;
+      settled[0] = lanes_any[0] == 0;
+      settled[1] = lanes_any[1] == 0;
       if (ntiles > 0) {
         int32_t a0, b0, a1, b1, a2, b2, a3, b3;  // blocks and counts of tiles t .. t+3
         uint32_t ca0, cb0, ca1, cb1, ca2, cb2, ca3, cb3;
@@ -540,6 +565,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
             if (4 * hh + 8 * (j >> 2) + (j & 3) > ragged_last) st[QT][j] = -INFINITY;
           pre(qt_tag, ragged_cnts, 0u);
           static_for<8>([&](auto j_tag) { exps(qt_tag, j_tag); });
+          exps_tail(qt_tag);
           static_for<4>([&](auto i_tag) { mma_pv(qt_tag, i_tag); });
         });
         exact = was_exact;
@@ -555,6 +581,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
           for (int r = 0; r < 16; r++) ot[dt][qt][r] = 0.f;
       m_i[0] = m_i[1] = -INFINITY;
       l_i[0] = l_i[1] = 0.f;
+      negm[0] = negm[1] = 0.f;
     }
   } else {
   const int nsteps = p.K;
