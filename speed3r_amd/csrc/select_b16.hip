@@ -72,6 +72,16 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
   char* k_buf[2] = {reinterpret_cast<char*>(lds_k0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_k1) + wave * kHalfBytes};
   char* v_buf[2] = {reinterpret_cast<char*>(lds_v0) + wave * kHalfBytes, reinterpret_cast<char*>(lds_v1) + wave * kHalfBytes};
 
+  // The four index rows of the group, one entry per lane.  They head the longest dependency chain of the start-up
+  // (rows -> walk list -> first tiles): their loads go first, ahead of the Q rows in the memory queue.
+  int32_t my_idx[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int qb = grp * 4 + j;
+    my_idx[j] = -1;
+    if (qb < nqb && lane < p.K) my_idx[j] = __builtin_nontemporal_load(p.idx + ((int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim + lane));
+  }
+  __builtin_amdgcn_sched_barrier(0);
   // B operand Q: lane = query row, head_dim chunk hh + 2 ks
   V8 bq[2][4];
 #pragma unroll
@@ -85,15 +95,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       bq[qt][ks] = as_v8<E>(f);
     }
   }
-  // the four index rows of the group, one entry per lane
-  int32_t my_idx[4];
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int qb = grp * 4 + j;
-    my_idx[j] = -1;
-    if (qb < nqb && lane < p.K) my_idx[j] = p.idx[(int64_t)b * p.sib + (int64_t)h * p.sih + (int64_t)qb * p.sim + lane];
+  for (int j = 0; j < 4; j++)
     if (my_idx[j] < 0 || (int64_t)my_idx[j] * 16 >= N) my_idx[j] = -1;
-  }
 
   f32x16 ot[2][2];  // O^T [dt][qt]
 #pragma unroll
@@ -232,10 +236,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     // whose block lists A (B) uses its 16 scores against A (B).  The visiting order differs from the lists' order,
     // which changes fp32 summation order only.
     //
-    // 1. The walk list is built first, in registers: entry n (lane n & 63 of register n >> 6) holds a distinct block
-    //    and four count bytes (how often query block j lists it; 0: not at all, above 1: a duplicated entry, which
-    //    attends the block that often).  One step takes the first remaining entry of any list (one ballot, three
-    //    selects), removes the block from all four lists and counts it (four compares).
+    // 1. The walk list is built first, in LDS: entry n holds a distinct block and four count bytes (how often query
+    //    block j lists it; 0: not at all, above 1: a duplicated entry, which attends the block that often).
     // 2. A software pipeline over units (tile t, half h of the 64 queries) then walks the list.  While the
     //    exponentials of unit u run on the VALU, the matrix pipe takes the scores of unit u + 1 and the PV product of
     //    unit u - 1, one MFMA per two exponentials.  K and V tiles come by direct transfers into two half buffers
@@ -250,34 +252,54 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     const int32_t ragged_blk = (N & 15) ? (int32_t)(N >> 4) : -2;  // the block that ends before its 16th row ...
     const int ragged_last = (int)(N & 15) - 1;
     uint32_t ragged_cnts = 0;  // ... stays out of the list: it gets a step of its own after the pipeline
+    // The distinct blocks and their counts come from a hash table in LDS (512 slots in the first K buffer, which
+    // the pipeline does not touch before the list is complete): every lane inserts its entry of list j with a
+    // compare-and-swap on the key (linear probing; at most 256 distinct blocks) and adds 1 << 8j to the slot's count;
+    // then the occupied slots are compacted into the list, eight slots per lane, positions from ballots.  The list's
+    // order is the table's, which is as good as any.
     int n_union = 0;
     uint32_t cnt_bits = 0;
     {
-      bool alive[4];
+      int32_t* const hkey = reinterpret_cast<int32_t*>(k_buf[0]);          // [512]
+      uint32_t* const hcnt = reinterpret_cast<uint32_t*>(k_buf[0] + 2048);  // [512]
+      reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
+      reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
+      reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
+      reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
 #pragma unroll
-      for (int j = 0; j < 4; j++) alive[j] = my_idx[j] >= 0;
-      while (true) {
-        const uint64_t any = __ballot(alive[0] || alive[1] || alive[2] || alive[3]);
-        if (any == 0) break;
-        const int i = __ffsll((unsigned long long)any) - 1;
-        const int32_t front = alive[0] ? my_idx[0] : alive[1] ? my_idx[1] : alive[2] ? my_idx[2] : my_idx[3];
-        const int32_t blk = __builtin_amdgcn_readlane(front, i);
-        uint32_t cnts = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {  // entries equal to blk are all still there: a block leaves all lists at once
-          const bool hit = my_idx[j] == blk;
-          cnts |= (uint32_t)__popcll(__ballot(hit)) << (8 * j);
-          alive[j] = alive[j] && !hit;
-        }
-        cnt_bits |= cnts;
-        if (blk == ragged_blk) {
-          ragged_cnts = cnts;
-        } else {
-          walk[n_union] = make_int2(blk, (int32_t)cnts);  // every lane writes the same pair
-          n_union++;
+      for (int j = 0; j < 4; j++) {
+        const int32_t e = my_idx[j];
+        ragged_cnts |= (uint32_t)__popcll(__ballot(e == ragged_blk)) << (8 * j);
+        bool active = e >= 0 && e != ragged_blk;
+        uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
+        while (active) {
+          const int32_t old = atomicCAS(hkey + slot, -1, e);
+          if (old == -1 || old == e) {
+            atomicAdd(hcnt + slot, 1u << (8 * j));
+            active = false;
+          } else {
+            slot = (slot + 1) & 511u;
+          }
         }
       }
-      walk[n_union] = make_int2(-1, 0);
+      const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
+      const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
+      const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+      const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      uint32_t pos = 0;  // occupied slots of the lanes below
+#pragma unroll
+      for (int s8 = 0; s8 < 8; s8++) {
+        const uint64_t m = __ballot(ks8[s8] >= 0);
+        pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
+        n_union += __popcll(m);
+        cnt_bits |= (uint32_t)cs8[s8];
+      }
+#pragma unroll
+      for (int s8 = 0; s8 < 8; s8++)
+        if (ks8[s8] >= 0) walk[pos++] = make_int2(ks8[s8], cs8[s8]);
+      if (lane == 0) walk[n_union] = make_int2(-1, 0);
+      cnt_bits = __any((cnt_bits & 0xfefefefeu) != 0) ? 2u : 0u;
+      cnt_bits |= ragged_cnts;
     }
     const bool dup = (cnt_bits & 0xfefefefeu) != 0;  // some list names a block more than once (wave-uniform)
     // tile tau = entries 2 tau, 2 tau + 1 of the walk list (-1 / no counts beyond its end): the read is issued early
