@@ -524,7 +524,9 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
 
-  float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight
+  float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight, as loaded
+  float staged_by = 1.f;       // the factor it is published with
+  bool staged_inf = false;     // BLK 16: rows past the end of a block publish lse = +inf
   float* staged_to = nullptr;  // where it goes in LDS
   // One query tile (64 rows of Q and dO, 64 lse and delta values) -> buffer BUF; each wave moves half of every
   // operand (instructions 2*wave, 2*wave+1 of both 32-row halves), wave 0 the lse values, wave 1 delta.
@@ -544,7 +546,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
       // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
       const int r = lane < last ? lane : last;
-      staged = ((wave == 0 ? lsep : dlp) + start)[r] * (wave == 0 ? kLog2e : scale);
+      staged = ((wave == 0 ? lsep : dlp) + start)[r];
+      staged_by = wave == 0 ? kLog2e : scale;
       staged_to = sb + 64 * wave + lane;
     } else {
       // this wave's half of the tile: the 16 queries of entries 2t and 2t + 1 of the current list (past its end: any
@@ -562,13 +565,17 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       const bool second = (j >> 4) != 0;
       const int nmine = second ? nb : na;
       const int64_t row = (second ? sbk : sa) + (j16 < nmine ? j16 : 0);
-      const float val = (hh == 0 ? lsep : dlp)[row] * (hh == 0 ? kLog2e : scale);
-      staged = (hh == 0 && j16 >= nmine) ? INFINITY : val;
+      staged = (hh == 0 ? lsep : dlp)[row];
+      staged_by = hh == 0 ? kLog2e : scale;
+      staged_inf = hh == 0 && j16 >= nmine;
       staged_to = sb + 64 * hh + 32 * wave + j;
     }
   };
+  // The loaded value is first touched here, a whole tile of work after its load: any arithmetic on it inside `fetch`
+  // would make the wave wait for the load there, and with it (the counter is in order) for the tile transfers issued
+  // just before, which is the tile that should be in flight during the current tile's work.
   auto publish = [&]() {
-    if (staged_to != nullptr) *staged_to = staged;
+    if (staged_to != nullptr) *staged_to = staged_inf ? INFINITY : staged * staged_by;
     staged_to = nullptr;
   };
   // One tile in three stages per 32-query half, issued so that the matrix products of one half run under the

@@ -504,7 +504,9 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
                  // three groups in four end here (16 266 keys, top-16: 1.11 -> 0.92 ms; 4 164 keys: 0.166 -> 0.152 ms); a
                  // second test over eight registers in front of this one gains 2 % more and is not worth its code.
                 const int kt = g / (16 / kGroup), r = (g % (16 / kGroup)) * kGroup;
-                const float m4 = fmaxf(fmaxf(st[kt][r], st[kt][r + 1]), fmaxf(st[kt][r + 2], st[kt][r + 3]));
+                float m4;  // two instructions by hand: the compiler's fmaxf quiets every operand first (a NaN loses either way)
+                asm("v_max3_f32 %0, %1, %2, %3\n\tv_max_f32 %0, %0, %4"
+                    : "=&v"(m4) : "v"(st[kt][r]), "v"(st[kt][r + 1]), "v"(st[kt][r + 2]), "v"(st[kt][r + 3]));
                 if (__builtin_amdgcn_ballot_w64(m4 >= thr) == 0) continue;
               }
 #pragma unroll
@@ -554,6 +556,9 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       }
       thr0 = qvalid ? tau : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
       thr = thr0;
+#ifdef S3R_IDX_NOSURV
+      thr = INFINITY;
+#endif
     }
     // Second sweep: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
     // through the lane's queue into its exact list.
