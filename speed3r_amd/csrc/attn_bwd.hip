@@ -131,6 +131,14 @@ __device__ __forceinline__ void read_rows(const char* half, int c, int hh, typen
   }
 }
 
+template <typename E, bool VSW>
+__device__ __forceinline__ typename Mma<E>::V8 read_row_frag(const char* half, int c, int hh, int ks) {
+  const int sw = VSW ? tsw(c) : (c & 7);
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(half + c * 128 + (((2 * ks + hh) ^ sw) << 4));
+  return as_v8<E>(f);
+}
+
 // A operand X^T from transposed reads of a half tile staged with VSW: fragment [jj][dt] holds, for head_dim row
 // dt*32 + c, the 8 rows 16jj + {4hh..4hh+3, 8+4hh..8+4hh+3} of the half: the order in which a 32x32 accumulator
 // with one column per lane hands over its registers 8jj .. 8jj+7.
@@ -146,6 +154,15 @@ __device__ __forceinline__ void read_transposed(const char* half, int tr_off, ty
       f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
       dst[jj][dt] = as_v8<E>(f);
     }
+}
+
+template <typename E>
+__device__ __forceinline__ typename Mma<E>::V8 read_transposed_frag(const char* half, int tr_off, int jj, int dt) {
+  const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+  Frag f;
+  f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+  f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+  return as_v8<E>(f);
 }
 
 __device__ __forceinline__ int tr_offset(int lane) {
@@ -523,6 +540,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const float sl2 = scale * kLog2e;
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
+  const uint32_t q_voff = (uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ tsw(lane >> 3)) * 16);
+  const uint32_t g_voff = (uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ tsw(lane >> 3)) * 16);
 
   float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight, as loaded
   float staged_by = 1.f;       // the factor it is published with
@@ -538,16 +557,35 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     if constexpr (BLK == 64) {
       const int64_t start = qblk * 64;
       const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
+      if (last >= 63) {
+        // (wave-uniform) a full tile: one per-lane offset per tensor (row lane/8 and its chunk; the chunk map only looks
+        // at the row's low three bits), the instruction's rows ride in the scalar offset
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + start * p.sqm), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + start * p.sgm), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
-      for (int hf = 0; hf < 2; hf++) {
-        dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * hf, last, qb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
-        dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+          for (int ii = 0; ii < 2; ii++) {
+            const int i = 2 * wave + ii;
+            const uint32_t rows = (uint32_t)(32 * hf + 8 * i);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (__attribute__((address_space(3))) void*)(qb + hf * kHalfBytes + i * 1024), 16,
+                                                     q_voff, rows * qrow, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rg, (__attribute__((address_space(3))) void*)(gb + hf * kHalfBytes + i * 1024), 16,
+                                                     g_voff, rows * grow, 0, 0);
+          }
+      } else {
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+          dma_rows<E, true>(qp + start * p.sqm, qrow, 32 * hf, last, qb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+          dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
+        }
       }
       // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
       // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
       const int r = lane < last ? lane : last;
       staged = ((wave == 0 ? lsep : dlp) + start)[r];
       staged_by = wave == 0 ? kLog2e : scale;
+      staged_inf = wave == 0 && lane > last;  // query rows beyond Lq: lse = +inf, no probability
       staged_to = sb + 64 * wave + lane;
     } else {
       // this wave's half of the tile: the 16 queries of entries 2t and 2t + 1 of the current list (past its end: any
@@ -641,16 +679,80 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         dkt[dt] = Mma<E>::mma(qt[jj][dt], db[jj], dkt[dt]);
       }
   };
+  // BLK 64: the same three stages with every instruction placed by hand, as in the forward kernel.  The vector work of
+  // a 32-query half (16 scores per lane: P, dS, their roundings) is cut into eight slots of two scores; each slot also
+  // issues one matrix product of another stage: the scores of half 1 run under the vector work of half 0, the dV / dK
+  // products of half 0 under the vector work of half 1.  Only the scores of half 0 and the products of half 1 have no
+  // vector work to hide behind.  Query rows beyond Lq need no masks: their lse is +inf.
+  auto tile64 = [&](auto bufc) {
+    constexpr int BUF = decltype(bufc)::value;
+    const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1);
+    const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1);
+    const float* sb = BUF == 0 ? lds_s0 : lds_s1;
+    f32x16 sc[2], dpv[2];   // S and dP of the two halves
+    V8 pbv[2][2], dbv[2][2];  // P and dS as B operands [half][jj]
+    V8 aq[4], ag[4];          // row fragments of Q, dO (A operands of the scores)
+    V8 gt[2][2], qt[2][2];    // transposed fragments of dO, Q (A operands of dV^T, dK^T)
+    auto mma_a = [&](auto hf_tag, auto i_tag) {  // product i of 8 of a half's scores: 0-3 S, 4-7 dP
+      constexpr int HF = decltype(hf_tag)::value, i = decltype(i_tag)::value, ks = i & 3;
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; r++) z[r] = 0.f;
+      if constexpr (i < 4) sc[HF] = Mma<E>::mma(aq[ks], bk[ks], ks == 0 ? z : sc[HF]);
+      else dpv[HF] = Mma<E>::mma(ag[ks], bv[ks], ks == 0 ? z : dpv[HF]);
+    };
+    auto mma_c = [&](auto hf_tag, auto i_tag) {  // product i of 8 of a half's dV^T / dK^T updates
+      constexpr int HF = decltype(hf_tag)::value, i = decltype(i_tag)::value, jj = (i >> 1) & 1, dt = i & 1;
+      if constexpr (i < 4) dvt[dt] = Mma<E>::mma(gt[jj][dt], pbv[HF][jj], dvt[dt]);
+      else dkt[dt] = Mma<E>::mma(qt[jj][dt], dbv[HF][jj], dkt[dt]);
+    };
+    auto vec = [&](auto hf_tag, auto j_tag) {  // scores 2j, 2j+1 of the half: P, dS, both rounded
+      constexpr int HF = decltype(hf_tag)::value, j = decltype(j_tag)::value, r = 2 * j;
+      // queries 4hh + 8(j/2) + 2(j%2) + {0, 1} of the half
+      const float2 l2 = *reinterpret_cast<const float2*>(sb + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
+      const float2 d2 = *reinterpret_cast<const float2*>(sb + 64 + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
+      f32x16& sh = sc[HF];
+      f32x16& dh = dpv[HF];
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(sh[r], sl2, -l2.x));
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(sh[r + 1], sl2, -l2.y));
+      const float e0 = p0 * fmaf(dh[r], scale, -d2.x);
+      const float e1 = p1 * fmaf(dh[r + 1], scale, -d2.y);
+      V8& pv = pbv[HF][r >> 3];
+      V8& dv = dbv[HF][r >> 3];
+      pv[r & 7] = (E)p0;
+      pv[(r & 7) + 1] = (E)p1;
+      dv[r & 7] = (E)e0;
+      dv[(r & 7) + 1] = (E)e1;
+    };
+    read_rows<E, true>(qb, c, hh, aq);
+    read_rows<E, true>(gb, c, hh, ag);
+    static_for<8>([&](auto i_tag) { mma_a(H0{}, i_tag); });
+    __builtin_amdgcn_sched_barrier(0);
+    // the fragments of a region's second four products are requested four slots ahead, one per slot, so that at most
+    // five fragments are in registers at a time
+    read_rows<E, true>(qb + kHalfBytes, c, hh, aq);
+    static_for<8>([&](auto j_tag) {
+      constexpr int j = decltype(j_tag)::value;
+      if constexpr (j < 4) ag[j] = read_row_frag<E, true>(gb + kHalfBytes, c, hh, j);
+      mma_a(H1{}, j_tag);
+      vec(H0{}, j_tag);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    read_transposed<E>(gb, tr_off, gt);
+    static_for<8>([&](auto j_tag) {
+      constexpr int j = decltype(j_tag)::value;
+      if constexpr (j < 4) qt[(j >> 1) & 1][j & 1] = read_transposed_frag<E>(qb, tr_off, (j >> 1) & 1, j & 1);
+      mma_c(H0{}, j_tag);
+      vec(H1{}, j_tag);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    read_transposed<E>(gb + kHalfBytes, tr_off, gt);
+    read_transposed<E>(qb + kHalfBytes, tr_off, qt);
+    static_for<8>([&](auto i_tag) { mma_c(H1{}, i_tag); });
+  };
   auto compute_tile = [&](int64_t qblk, auto bufc) {
     if constexpr (BLK == 64) {
-      f32x16 s0, dp0, s1, dp1;
-      V8 pb0[2], db0[2], pb1[2], db1[2];
-      stage_a(bufc, 0, s0, dp0);
-      stage_a(bufc, 1, s1, dp1);
-      stage_b(qblk, bufc, 0, s0, dp0, pb0, db0);
-      stage_c(bufc, 0, pb0, db0);
-      stage_b(qblk, bufc, 1, s1, dp1, pb1, db1);
-      stage_c(bufc, 1, pb1, db1);
+      tile64(bufc);
     } else {  // this wave's keys only meet the queries of its own half of the tile
       f32x16 s0, dp0;
       V8 pb0[2], db0[2];
