@@ -48,6 +48,16 @@ def test_host_side_validation_returns_error_codes():
                                       _lib.S3R_BF16, None) == -2                                    # K not a power of two
     assert L.s3r_gated_merge(ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16),
                              1, 1, 64, 64, 64, *([0] * 9), 7, None) == -2                           # unknown dtype
+    one = ctypes.c_void_p(16)
+
+    def causal(o=one, idx=one, scores=one, k=8, d=64):
+        return L.s3r_compressed_attn_topk_causal(one, one, one, o, None, idx, scores, 1, 1, 8, 8, d, k, *([0] * 12),
+                                                 0.125, _lib.S3R_BF16, None)
+
+    assert causal(o=None) == _lib.S3R_ERR_BAD_ARG                    # the causal entry always writes o
+    assert causal(scores=None) == _lib.S3R_ERR_BAD_ARG               # its indices are selected from the score buffer
+    assert b"score buffer" in L.s3r_last_error()
+    assert causal(k=12) == _lib.S3R_ERR_UNSUPPORTED and causal(d=128) == _lib.S3R_ERR_UNSUPPORTED
 
 
 def test_backward_entry_points_validate_on_the_host():
