@@ -93,28 +93,26 @@ template <int N> __device__ __forceinline__ void bitonic_merge_desc(key_t (&x)[N
     for (int i = 0; i < N; i++)
       if ((i & d) == 0) cex_desc(x[i], x[i | d]);
 }
-template <int N> __device__ __forceinline__ void bitonic_sort_desc(key_t (&x)[N]) {
+// top-N of (descending a) U (descending b) -> a, descending; the last NF entries of b are fillers (key 0, below
+// every real key), so the first NF entries of a meet nothing
+template <int N, int NF = 0> __device__ __forceinline__ void merge_top_desc(key_t (&a)[N], const key_t (&b)[N]) {
 #pragma unroll
-  for (int k = 2; k <= N; k <<= 1)
-#pragma unroll
-    for (int d = k / 2; d >= 1; d >>= 1)
-#pragma unroll
-      for (int i = 0; i < N; i++) {
-        const int j = i ^ d;
-        if (j > i) {
-          if ((i & k) == 0 || k == N) {  // descending run (the last stage sorts everything descending)
-            cex_desc(x[i], x[j]);
-          } else {  // ascending run
-            cex_desc(x[j], x[i]);
-          }
-        }
-      }
-}
-// top-N of (descending a) U (descending b) -> a, descending
-template <int N> __device__ __forceinline__ void merge_top_desc(key_t (&a)[N], const key_t (&b)[N]) {
-#pragma unroll
-  for (int i = 0; i < N; i++) a[i] = __builtin_fmax(a[i], b[N - 1 - i]);  // half-cleaner: a is now bitonic
+  for (int i = NF; i < N; i++) a[i] = __builtin_fmax(a[i], b[N - 1 - i]);  // half-cleaner: a is now bitonic
   bitonic_merge_desc<N>(a);
+}
+// Sorting network for the 13 entries a lane's queue can hold (descending, entries 0..12 of x): Batcher's odd-even
+// merge sort for 16 inputs without the comparators that touch inputs 13..15, 48 compare-exchanges against the 80
+// of the bitonic network for 16 (checked on all 2^13 zero-one inputs by tests/test_sort_network.py).
+constexpr int kSortNet13Size = 48;
+constexpr signed char kSortNet13[kSortNet13Size][2] = {
+    {0, 1}, {2, 3}, {0, 2}, {1, 3}, {1, 2}, {4, 5}, {6, 7}, {4, 6}, {5, 7}, {5, 6}, {0, 4}, {2, 6},
+    {2, 4}, {1, 5}, {3, 7}, {3, 5}, {1, 2}, {3, 4}, {5, 6}, {8, 9}, {10, 11}, {8, 10}, {9, 11}, {9, 10},
+    {8, 12}, {10, 12}, {9, 10}, {11, 12}, {0, 8}, {4, 12}, {4, 8}, {2, 10}, {6, 10}, {2, 4}, {6, 8}, {10, 12},
+    {1, 9}, {5, 9}, {3, 11}, {7, 11}, {3, 5}, {7, 9}, {1, 2}, {3, 4}, {5, 6}, {7, 8}, {9, 10}, {11, 12}};
+template <int N> __device__ __forceinline__ void sort13_desc(key_t (&x)[N]) {
+  static_assert(N >= 13, "the network sorts entries 0..12");
+#pragma unroll
+  for (int i = 0; i < kSortNet13Size; i++) cex_desc(x[kSortNet13[i][0]], x[kSortNet13[i][1]]);
 }
 
 constexpr int kTile = 64 * 64;  // elements per LDS tile
@@ -140,6 +138,12 @@ template <> struct TopkCfg<0> {
 template <int OFF> __device__ __forceinline__ u32x4 lds_read16_async(uint32_t addr) {
   u32x4 v;
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <int OFF> __device__ __forceinline__ u32x2 lds_read8_async(uint32_t addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
 }
 __device__ __forceinline__ void lds_reads_done(u32x4 (&a)[2][4]) {
@@ -230,25 +234,42 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
   const uint32_t lkm1 = (uint32_t)(Lk - 1);
 
   auto drain = [&]() {  // merge this lane's queue into its list; every lane runs the same network
+    // Lists up to 16 entries: all queue slots are fetched at once and waited for once (hand-written reads: left to the
+    // compiler, each read lands inside the `e < qn` branch of its entry with a wait of its own, thirteen LDS round
+    // trips in a row; top-16 at 4 164 keys 0.148 -> 0.140 ms).  The top-32 instance has no registers for that.
+    constexpr bool kPrefetch = KL <= 16;
+    u32x2 raw[kQSlots > 1 ? kQSlots - 1 : 1];  // (the attention instance has no queue and never folds)
+    if constexpr (kPrefetch) {
+      const uint32_t qaddr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(qlane);
+#pragma unroll
+      for (int e = 0; e < kQSlots - 1; e++) raw[e] = lds_read8_async<0>(qaddr + e * 64 * 8);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
     key_t cand[kQCap];
 #pragma unroll
     for (int e = 0; e < kQCap; e++) {
       cand[e] = 0;
       if (e < kQSlots - 1) {
-        const uint2 v = qlane[e * 64];
-        cand[e] = e < qn ? make_key(v.x, lkm1 - v.y) : 0.0;
+        if constexpr (kPrefetch) {
+          asm volatile("" : "+v"(raw[e]));  // the value exists from here on, whatever the branch below does
+          cand[e] = e < qn ? make_key(raw[e][0], lkm1 - raw[e][1]) : 0.0;
+        } else {
+          const uint2 v = qlane[e * 64];
+          cand[e] = e < qn ? make_key(v.x, lkm1 - v.y) : 0.0;
+        }
       }
     }
-    bitonic_sort_desc<kQCap>(cand);
+    // the queue's 13 entries through their own network; cand[13..15] stay fillers
+    static_assert(!FUSED || (kQSlots - 1 == 13 && kQCap == 16), "the fold is built for 13 queue entries in a 16-wide merge");
+    constexpr int kFill = kQCap - 13;
+    sort13_desc(cand);
     if constexpr (KL == kQCap) {
-      merge_top_desc<KL>(list, cand);
-    } else if constexpr (KL < kQCap) {  // keep the KL best of list U cand: widen the list, merge, truncate
-      key_t wide[kQCap];
+      merge_top_desc<KL, kFill>(list, cand);
+    } else if constexpr (KL < kQCap) {  // the KL best of list U cand are among the list and the KL best candidates
+      key_t best[KL];
 #pragma unroll
-      for (int i = 0; i < kQCap; i++) wide[i] = i < KL ? list[i] : 0;
-      merge_top_desc<kQCap>(wide, cand);
-#pragma unroll
-      for (int i = 0; i < KL; i++) list[i] = wide[i];
+      for (int i = 0; i < KL; i++) best[i] = cand[i];
+      merge_top_desc<KL>(list, best);
     } else {  // KL == 2 * kQCap, in place: the upper half U of the list beats its lower half M, and an element of
       // M U cand outside that set's best kQCap cannot be among the KL best of the whole (kQCap of that set and, being
       // below all of U, all kQCap of U are above it).  So: lower half <- best kQCap of M U cand, then one bitonic
@@ -257,7 +278,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       key_t lower[kQCap];
 #pragma unroll
       for (int i = 0; i < kQCap; i++) lower[i] = list[kQCap + i];
-      merge_top_desc<kQCap>(lower, cand);
+      merge_top_desc<kQCap, kFill>(lower, cand);
 #pragma unroll
       for (int i = 0; i < kQCap; i++) list[kQCap + i] = lower[kQCap - 1 - i];  // descending, then ascending: bitonic
       bitonic_merge_desc<KL>(list);
@@ -412,21 +433,29 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     // the tile being read; wave w moves rows 16w .. 16w+15 of a tile (two instructions of 8 rows).  LDS chunk
     // (row, c') holds head_dim chunk c' ^ (row & 7).  Rows beyond Lk re-read the last row (they are masked).
     const uint32_t krow_bytes = (uint32_t)p.skn * (uint32_t)sizeof(E);
-    const int dl_row = wave * 16 + (lane >> 3);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the LDS destination of a transfer is a scalar (M0)
+    const int dl_row = wave_u * 16 + (lane >> 3);
     const uint32_t dl_chunk = (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
+    const uint32_t dl_off[2] = {(uint32_t)dl_row * krow_bytes + dl_chunk, (uint32_t)(dl_row + 8) * krow_bytes + dl_chunk};
     auto dma_tile = [&](int t, int buf) {  // tiles past the end repeat the last one (never read)
       const int tt = t < ntiles ? t : ntiles - 1;
       const int64_t start = (int64_t)tt * 64;
       const int rem = (int)(Lk - 1 - start);
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
-      char* dst = reinterpret_cast<char*>(&Ks[buf][0]) + wave * 2048;
+      char* dst = reinterpret_cast<char*>(&Ks[buf][0]) + wave_u * 2048;
+      uint32_t off[2] = {dl_off[0], dl_off[1]};  // the per-lane offsets of a full tile never change
+      if (__builtin_expect(rem < 63, 0)) {       // ragged last tile: rows beyond the end re-read the last row
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        int r = dl_row + 8 * i;
-        r = r < rem ? r : rem;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16,
-                                                 (uint32_t)r * krow_bytes + dl_chunk, 0, 0, 0);
+        for (int i = 0; i < 2; i++) {
+          int r = dl_row + 8 * i;
+          r = r < rem ? r : rem;
+          off[i] = (uint32_t)r * krow_bytes + dl_chunk;
+          asm volatile("" : "+v"(off[i]));       // stays inside this branch
+        }
       }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, off[i], 0, 0, 0);
     };
     const uint32_t lds_k = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(&Ks[0][0]);
     const uint32_t kr_off = lds_k + (uint32_t)(c * 128 + ((hh ^ (c & 7)) << 4));  // A operand: lane = key row, chunk hh + 2 ks
