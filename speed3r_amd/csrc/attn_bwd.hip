@@ -75,14 +75,9 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const E* __restrict__ o,
 
 // ---- shared pieces of the two MFMA kernels -----------------------------------------------------------------------
 // Transfer of rows [8*i0*.., ...) of a 32-row half tile: instruction i moves rows 8i .. 8i+7 (16 bytes per lane).
-// VSW: LDS chunk (row, c') holds head_dim chunk c' ^ tsw(row), tsw(row) = bit2 | (bit0 ^ bit1) << 1 | bit1 << 2 of the
-// row: of the 32768 GF(2)-linear maps from the 5 row bits to the 3 chunk bits, timed on the device, this is one of
-// those whose 16-byte row reads AND ds_read_b64_tr_b16 reads both run without bank conflicts (the transposed reads
-// take 1.3x as long with the plain (row & 7) map or none), and it only looks at row bits 0..2, so rows 8 and 16
-// further down keep the same map.  Otherwise c' ^ (row & 7) (row reads only).  Rows are clamped to `last`
-// (relative to `base`'s row 0).
-__device__ __forceinline__ int tsw(int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ row) & 1) << 1) | (((row >> 1) & 1) << 2); }
-
+// LDS chunk (row, c') holds head_dim chunk c' ^ k_swizzle(row) in every tile: 16-byte row reads and
+// ds_read_b64_tr_b16 reads both run without bank conflicts with it.  (VSW marks the tiles that are also read
+// transposed; the map is the same.)  Rows are clamped to `last` (relative to `base`'s row 0).
 template <typename E, bool VSW>
 __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int first_row, int last, char* lds_half, int lane, int i_begin, int i_end) {
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
@@ -93,7 +88,7 @@ __device__ __forceinline__ void dma_rows(const E* base, uint32_t rowbytes, int f
       const int ldsrow = 8 * i + lr;
       int row = first_row + ldsrow;
       row = row < last ? row : last;
-      const int chunk = (lane & 7) ^ (VSW ? tsw(ldsrow) : (ldsrow & 7));
+      const int chunk = (lane & 7) ^ k_swizzle(ldsrow);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
                                                (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
     }
@@ -113,7 +108,7 @@ __device__ __forceinline__ void dma_rows16(const E* base_a, const E* base_b, uin
     const int last = i < 2 ? last_a : last_b;
     int row = ldsrow & 15;
     row = row < last ? row : last;
-    const int chunk = (lane & 7) ^ (VSW ? tsw(ldsrow) : (ldsrow & 7));
+    const int chunk = (lane & 7) ^ k_swizzle(ldsrow);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? ra : rb, (__attribute__((address_space(3))) void*)(lds_half + i * 1024), 16,
                                              (uint32_t)row * rowbytes + (uint32_t)(chunk * 16), 0, 0, 0);
   }
@@ -122,7 +117,7 @@ __device__ __forceinline__ void dma_rows16(const E* base_a, const E* base_b, uin
 // A operand from row reads of a half tile: lane = row c, k-step ks: head_dim chunk 2ks + hh.
 template <typename E, bool VSW>
 __device__ __forceinline__ void read_rows(const char* half, int c, int hh, typename Mma<E>::V8 (&dst)[4]) {
-  const int sw = VSW ? tsw(c) : (c & 7);
+  const int sw = k_swizzle(c);
 #pragma unroll
   for (int ks = 0; ks < 4; ks++) {
     Frag f;
@@ -133,7 +128,7 @@ __device__ __forceinline__ void read_rows(const char* half, int c, int hh, typen
 
 template <typename E, bool VSW>
 __device__ __forceinline__ typename Mma<E>::V8 read_row_frag(const char* half, int c, int hh, int ks) {
-  const int sw = VSW ? tsw(c) : (c & 7);
+  const int sw = k_swizzle(c);
   Frag f;
   f.u = *reinterpret_cast<const uint4*>(half + c * 128 + (((2 * ks + hh) ^ sw) << 4));
   return as_v8<E>(f);
@@ -149,9 +144,10 @@ __device__ __forceinline__ void read_transposed(const char* half, int tr_off, ty
 #pragma unroll
     for (int dt = 0; dt < 2; dt++) {
       const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+      const char* a8 = half + (tr_off ^ (dt * 64) ^ 64) + (jj * 16 + 8) * 128;  // rows 8 further down: chunk map ^ 4
       Frag f;
       f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
-      f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+      f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a8));
       dst[jj][dt] = as_v8<E>(f);
     }
 }
@@ -159,9 +155,10 @@ __device__ __forceinline__ void read_transposed(const char* half, int tr_off, ty
 template <typename E>
 __device__ __forceinline__ typename Mma<E>::V8 read_transposed_frag(const char* half, int tr_off, int jj, int dt) {
   const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
+  const char* a8 = half + (tr_off ^ (dt * 64) ^ 64) + (jj * 16 + 8) * 128;
   Frag f;
   f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
-  f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * 128));
+  f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a8));
   return as_v8<E>(f);
 }
 
@@ -169,7 +166,7 @@ __device__ __forceinline__ int tr_offset(int lane) {
   const int hh = lane >> 5;
   const int i16 = lane & 15;
   const int tr_row = 4 * hh + (i16 >> 2);
-  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ tsw(tr_row);
+  const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ k_swizzle(tr_row);
   return tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
 }
 
@@ -540,8 +537,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const float sl2 = scale * kLog2e;
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
-  const uint32_t q_voff = (uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ tsw(lane >> 3)) * 16);
-  const uint32_t g_voff = (uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ tsw(lane >> 3)) * 16);
+  // (one per parity of the instruction inside its half tile: the chunk map of rows 8..15 differs from that of rows 0..7)
+  const uint32_t q_voff[2] = {(uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16),
+                              (uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
+  const uint32_t g_voff[2] = {(uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16),
+                              (uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
 
   float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight, as loaded
   float staged_by = 1.f;       // the factor it is published with
@@ -558,8 +558,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       const int64_t start = qblk * 64;
       const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
       if (last >= 63) {
-        // (wave-uniform) a full tile: one per-lane offset per tensor (row lane/8 and its chunk; the chunk map only looks
-        // at the row's low three bits), the instruction's rows ride in the scalar offset
+        // (wave-uniform) a full tile: per-lane offsets (row lane/8 and its chunk) that do not depend on the tile, the
+        // instruction's rows ride in the scalar offset
         const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + start * p.sqm), 0, 0x7fffffff, 0x00020000);
         const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + start * p.sgm), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
@@ -569,9 +569,9 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
             const int i = 2 * wave + ii;
             const uint32_t rows = (uint32_t)(32 * hf + 8 * i);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (__attribute__((address_space(3))) void*)(qb + hf * kHalfBytes + i * 1024), 16,
-                                                     q_voff, rows * qrow, 0, 0);
+                                                     q_voff[ii], rows * qrow, 0, 0);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rg, (__attribute__((address_space(3))) void*)(gb + hf * kHalfBytes + i * 1024), 16,
-                                                     g_voff, rows * grow, 0, 0);
+                                                     g_voff[ii], rows * grow, 0, 0);
           }
       } else {
 #pragma unroll

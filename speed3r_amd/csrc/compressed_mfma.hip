@@ -6,7 +6,7 @@
 // tiles of 64 pooled tokens.  K and V tiles are staged once per workgroup in LDS (global ->
 // registers two tiles ahead -> LDS one tile ahead, two LDS buffers, one barrier per tile) and
 // shared by the four waves.  Rows are 128 bytes without padding; 16-byte chunks are stored
-// XOR-swizzled (K: chunk ^ (row & 7) for the 16-byte operand reads, V: halves swapped on rows
+// XOR-swizzled (K: chunk ^ ((row >> 1) & 7) for the 16-byte operand reads, V: halves swapped on rows
 // 2,3 mod 4 for the transposed reads) so that LDS reads are bank-conflict free.
 // Per wave and tile: S^T = K Q^T with v_mfma_f32_32x32x16 (one query per lane and its partner
 // lane ^ 32, 32 of the tile's 64 keys in each lane's registers), base-2 online softmax in
@@ -140,7 +140,6 @@ template <int OFF> __device__ __forceinline__ u32x4 lds_read16_async(uint32_t ad
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
 }
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 template <int OFF> __device__ __forceinline__ u32x2 lds_read8_async(uint32_t addr) {
   u32x2 v;
   asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
@@ -205,7 +204,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       const int r = ld_row + 32 * i;
       int64_t row = start + r;
       row = row < Lk ? row : Lk - 1;
-      kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ (r & 7)) * 8));
+      kr[i] = *reinterpret_cast<const uint4*>(kp + row * p.skn + ((ld_pos ^ k_swizzle(r)) * 8));
       vr[i] = *reinterpret_cast<const uint4*>(vp + row * p.svn + ((ld_pos ^ (((r >> 1) & 1) << 2)) * 8));
     }
   };
@@ -318,7 +317,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
         Frag f;
-        f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ (c & 7)) * 16));
+        f.u = *reinterpret_cast<const uint4*>(kbase + (kt * 32 + c) * 128 + (((ks * 2 + hh) ^ k_swizzle(c)) * 16));
         st[kt] = Mma<E>::mma(as_v8<E>(f), bq[ks], st[kt]);
       }
     }
@@ -431,12 +430,12 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     // One sweep over the key tiles: S^T by MFMA, then either the group maxima (first sweep) or the candidate filter
     // (second sweep).  K tiles go global -> LDS by direct transfers into a ring of NB buffers, NB - 1 tiles ahead of
     // the tile being read; wave w moves rows 16w .. 16w+15 of a tile (two instructions of 8 rows).  LDS chunk
-    // (row, c') holds head_dim chunk c' ^ (row & 7).  Rows beyond Lk re-read the last row (they are masked).
+    // (row, c') holds head_dim chunk c' ^ k_swizzle(row).  Rows beyond Lk re-read the last row (they are masked).
     const uint32_t krow_bytes = (uint32_t)p.skn * (uint32_t)sizeof(E);
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the LDS destination of a transfer is a scalar (M0)
     const int dl_row = wave_u * 16 + (lane >> 3);
-    const uint32_t dl_chunk = (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
-    const uint32_t dl_off[2] = {(uint32_t)dl_row * krow_bytes + dl_chunk, (uint32_t)(dl_row + 8) * krow_bytes + dl_chunk};
+    const uint32_t dl_chunk[2] = {(uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16), (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
+    const uint32_t dl_off[2] = {(uint32_t)dl_row * krow_bytes + dl_chunk[0], (uint32_t)(dl_row + 8) * krow_bytes + dl_chunk[1]};
     auto dma_tile = [&](int t, int buf) {  // tiles past the end repeat the last one (never read)
       const int tt = t < ntiles ? t : ntiles - 1;
       const int64_t start = (int64_t)tt * 64;
@@ -449,7 +448,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
         for (int i = 0; i < 2; i++) {
           int r = dl_row + 8 * i;
           r = r < rem ? r : rem;
-          off[i] = (uint32_t)r * krow_bytes + dl_chunk;
+          off[i] = (uint32_t)r * krow_bytes + dl_chunk[i];
           asm volatile("" : "+v"(off[i]));       // stays inside this branch
         }
       }
@@ -458,7 +457,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, off[i], 0, 0, 0);
     };
     const uint32_t lds_k = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(&Ks[0][0]);
-    const uint32_t kr_off = lds_k + (uint32_t)(c * 128 + ((hh ^ (c & 7)) << 4));  // A operand: lane = key row, chunk hh + 2 ks
+    const uint32_t kr_off = lds_k + (uint32_t)(c * 128 + ((hh ^ k_swizzle(c)) << 4));  // A operand: lane = key row, chunk hh + 2 ks
     auto sweep = [&](auto filter_tag, const int stride) {  // tiles 0, stride, 2 stride, ...
       constexpr bool FILTER = decltype(filter_tag)::value;
       const int nsteps = (ntiles + stride - 1) / stride;

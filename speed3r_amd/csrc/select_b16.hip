@@ -116,7 +116,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
   const int tr_row = 4 * hh + (i16 >> 2);
   const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
   const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
-  const int kr_off = c * 128 + ((hh ^ (c & 7)) << 4);
+  const int kr_off = c * 128 + ((hh ^ k_swizzle(c)) << 4);
 
   // Unit (i, QT): list position i of query blocks 2 QT and 2 QT + 1.  blk[0], blk[1]: their key blocks (-1: skip).
   auto entry = [&](int i, auto qt_tag, int32_t (&blk)[2]) {
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
         const int ldsrow = 16 * s + 8 * t + lr;   // row of the 32-row half tile
         int row = 8 * t + lr;                     // row of the 16-token block
         row = row < last ? row : last;
-        const uint32_t kc = (uint32_t)(((lane & 7) ^ (ldsrow & 7)) * 16);
+        const uint32_t kc = (uint32_t)(((lane & 7) ^ k_swizzle(ldsrow)) * 16);
         const uint32_t vc = (uint32_t)(((lane & 7) ^ (((ldsrow >> 1) & 1) << 2)) * 16);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(k_buf[QT] + (2 * s + t) * 1024), 16,
                                                  (uint32_t)row * krow + kc, 0, 0, 0);
@@ -318,24 +318,26 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     };
 
     // ---- transfers: one descriptor per tensor, the block's byte offset rides in the scalar offset ----
-    const uint32_t koff = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ lr) * 16);
+    // (the K swizzle of a block's rows 8..15 differs from that of its rows 0..7: one offset per instruction of a block)
+    const uint32_t koff = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ k_swizzle(lr)) * 16);
+    const uint32_t koff8 = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ k_swizzle(lr + 8)) * 16);
     const uint32_t voff = (uint32_t)lr * vrow + (uint32_t)(((lane & 7) ^ (((lr >> 1) & 1) << 2)) * 16);
     typedef __attribute__((address_space(3))) char* LdsPtr;  // arithmetic stays in the LDS address space (no null checks)
     const LdsPtr k_lds[2] = {(LdsPtr)lds_k0 + wave * kHalfBytes, (LdsPtr)lds_k1 + wave * kHalfBytes};
     const LdsPtr v_lds[2] = {(LdsPtr)lds_v0 + wave * kHalfBytes, (LdsPtr)lds_v1 + wave * kHalfBytes};
     // 16 rows of one block -> 2 KB at dst.  The instruction's immediate offset moves the LDS side and the global side
     // alike; the scalar offset makes up the difference (row strides are at least 128 bytes).
-    auto dma_block = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t rowb, int32_t blk) {
+    auto dma_block = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb, int32_t blk) {
       const uint32_t so = (uint32_t)blk * 16u * rowb;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off0, so, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off0, so + (8u * rowb - 1024u), 1024, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off8, so + (8u * rowb - 1024u), 1024, 0);
     };
-    auto dma_ragged = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t rowb) {  // rows beyond the sequence re-read its last row
+    auto dma_ragged = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb) {  // rows beyond the sequence re-read its last row
       const uint32_t so = (uint32_t)ragged_blk * 16u * rowb;
       const int r0 = lr < ragged_last ? lr : ragged_last, r1 = 8 + lr < ragged_last ? 8 + lr : ragged_last;
-      const uint32_t col = off0 - (uint32_t)lr * rowb;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (uint32_t)r0 * rowb + col, so, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst + 1024, 16, (uint32_t)r1 * rowb + col, so, 0, 0);
+      const uint32_t col0 = off0 - (uint32_t)lr * rowb, col8 = off8 - (uint32_t)lr * rowb;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (uint32_t)r0 * rowb + col0, so, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst + 1024, 16, (uint32_t)r1 * rowb + col8, so, 0, 0);
     };
     // A tile beyond the end of the list (a < 0) is requested all the same, through a descriptor of zero records:
     // every lane is out of range, nothing is fetched, and the count of outstanding transfers does not depend on the
@@ -348,14 +350,14 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     auto dma_k = [&](auto par_tag, int32_t a, int32_t b2) {
       constexpr int P = decltype(par_tag)::value;
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, records(a), 0x00020000);
-      dma_block(rs, k_lds[P], koff, krow, a);
-      dma_block(rs, k_lds[P] + 2048, koff, krow, b2 < 0 ? a : b2);
+      dma_block(rs, k_lds[P], koff, koff8, krow, a);
+      dma_block(rs, k_lds[P] + 2048, koff, koff8, krow, b2 < 0 ? a : b2);
     };
     auto dma_v = [&](auto par_tag, int32_t a, int32_t b2) {
       constexpr int P = decltype(par_tag)::value;
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, records(a), 0x00020000);
-      dma_block(rs, v_lds[P], voff, vrow, a);
-      dma_block(rs, v_lds[P] + 2048, voff, vrow, b2 < 0 ? a : b2);
+      dma_block(rs, v_lds[P], voff, voff, vrow, a);
+      dma_block(rs, v_lds[P] + 2048, voff, voff, vrow, b2 < 0 ? a : b2);
     };
     const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, -1, 0x00020000);
@@ -570,10 +572,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       }
       if (ragged_cnts != 0) {  // the block that ends the sequence early: one unpipelined step with the running maximum
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): earlier reads of the buffers are done
-        dma_ragged(rk, k_lds[0], koff, krow);
-        dma_ragged(rk, k_lds[0] + 2048, koff, krow);  // the tile's second block: the same rows again (finite values)
-        dma_ragged(rv, v_lds[0], voff, vrow);
-        dma_ragged(rv, v_lds[0] + 2048, voff, vrow);
+        dma_ragged(rk, k_lds[0], koff, koff8, krow);
+        dma_ragged(rk, k_lds[0] + 2048, koff, koff8, krow);  // the tile's second block: the same rows again (finite values)
+        dma_ragged(rv, v_lds[0], voff, voff, vrow);
+        dma_ragged(rv, v_lds[0] + 2048, voff, voff, vrow);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         load_k(H0{});
         load_v(H0{});

@@ -126,7 +126,6 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   // path a quarter of what operand-pattern global loads cost.  Rows beyond N re-read the last row (never stored).
   {
     const int qr = lane >> 3;
-    const uint32_t q_chunk = (uint32_t)(((lane & 7) ^ (qr & 7)) * 8 * (int)sizeof(E));
     const uint32_t q_rowbytes = (uint32_t)p.sqm * (uint32_t)sizeof(E);
     const int q_last = (int)((N - q0 < 64 ? N - q0 : 64) - 1);
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + q0 * p.sqm), 0, 0x7fffffff, 0x00020000);
@@ -138,7 +137,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         int row = 32 * qt + 8 * i + qr;
         row = row < q_last ? row : q_last;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16,
-                                                 (uint32_t)row * q_rowbytes + q_chunk, 0, 0, 2 /* nt: the Q block is read once */);
+                                                 (uint32_t)row * q_rowbytes + (uint32_t)(((lane & 7) ^ k_swizzle(8 * i + qr)) * 16), 0, 0,
+                                                 2 /* nt: the Q block is read once */);
       }
     }
   }
@@ -200,9 +200,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   V8 vfr[2][2];     // V^T fragments of one half tile [jj][dt]
 
   // ---- transfers global -> LDS (8 rows of 128 bytes per instruction, 16 bytes per lane) ----
-  // K: LDS chunk (row, c') holds head_dim chunk c' ^ (row & 7); V: chunks of rows 2,3 (mod 4) have their halves swapped
+  // K: LDS chunk (row, c') holds head_dim chunk c' ^ k_swizzle(row), which differs between the rows of an even and of an
+  // odd instruction of a tile; V: chunks of rows 2,3 (mod 4) have their halves swapped
   const int ld_row = lane >> 3;
-  const uint32_t k_voff = ((uint32_t)ld_row * (uint32_t)p.skn + (((lane & 7) ^ (ld_row & 7)) * 8)) * (uint32_t)sizeof(E);
+  const uint32_t k_voff[2] = {((uint32_t)ld_row * (uint32_t)p.skn + (((lane & 7) ^ k_swizzle(ld_row)) * 8)) * (uint32_t)sizeof(E),
+                              ((uint32_t)ld_row * (uint32_t)p.skn + (((lane & 7) ^ k_swizzle(ld_row + 8)) * 8)) * (uint32_t)sizeof(E)};
   const uint32_t v_voff = ((uint32_t)ld_row * (uint32_t)p.svn + (((lane & 7) ^ (((ld_row >> 1) & 1) << 2)) * 8)) * (uint32_t)sizeof(E);
   // the instruction's immediate offset moves the LDS side AND the global side by i KB: the scalar offset makes up the rest
   const uint32_t k_step = 8u * (uint32_t)p.skn * (uint32_t)sizeof(E) - 1024u;
@@ -211,10 +213,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     constexpr int HF = decltype(hf)::value;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + (start + 32 * HF) * p.skn), 0, 0x7fffffff, 0x00020000);
     __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)k_half(hf);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff, 0, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff, k_step, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff, 2 * k_step, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff, 3 * k_step, 3072, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[0], 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[1], k_step, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[0], 2 * k_step, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[1], 3 * k_step, 3072, 0);
   };
   auto dma_v = [&](auto hf, int64_t start) {
     constexpr int HF = decltype(hf)::value;
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   // can otherwise overtake a read still queued in the LDS pipeline)
   auto reads_done = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };  // lgkmcnt(0)
   // ---- LDS -> registers ----
-  const int kr_off = c * 128 + ((hh ^ (c & 7)) << 4);
+  const int kr_off = c * 128 + ((hh ^ k_swizzle(c)) << 4);
   auto read_k = [&](auto hf, V8 (&dst)[4]) {  // A operand: lane = key row, head_dim chunk hh + 2*ks
     const char* kbase = reinterpret_cast<const char*>(k_half(hf));
 #pragma unroll
