@@ -233,12 +233,11 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
   const uint32_t lkm1 = (uint32_t)(Lk - 1);
 
   auto drain = [&]() {  // merge this lane's queue into its list; every lane runs the same network
-    // Lists up to 16 entries: all queue slots are fetched at once and waited for once (hand-written reads: left to the
-    // compiler, each read lands inside the `e < qn` branch of its entry with a wait of its own, thirteen LDS round
-    // trips in a row; top-16 at 4 164 keys 0.148 -> 0.140 ms).  The top-32 instance has no registers for that.
-    constexpr bool kPrefetch = KL <= 16;
+    // All queue slots are fetched at once and waited for once (hand-written reads: left to the compiler, each read
+    // lands inside the `e < qn` branch of its entry with a wait of its own, thirteen LDS round trips in a row;
+    // top-16 at 4 164 keys 0.148 -> 0.140 ms).
     u32x2 raw[kQSlots > 1 ? kQSlots - 1 : 1];  // (the attention instance has no queue and never folds)
-    if constexpr (kPrefetch) {
+    {
       const uint32_t qaddr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(qlane);
 #pragma unroll
       for (int e = 0; e < kQSlots - 1; e++) raw[e] = lds_read8_async<0>(qaddr + e * 64 * 8);
@@ -249,13 +248,8 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     for (int e = 0; e < kQCap; e++) {
       cand[e] = 0;
       if (e < kQSlots - 1) {
-        if constexpr (kPrefetch) {
-          asm volatile("" : "+v"(raw[e]));  // the value exists from here on, whatever the branch below does
-          cand[e] = e < qn ? make_key(raw[e][0], lkm1 - raw[e][1]) : 0.0;
-        } else {
-          const uint2 v = qlane[e * 64];
-          cand[e] = e < qn ? make_key(v.x, lkm1 - v.y) : 0.0;
-        }
+        asm volatile("" : "+v"(raw[e]));  // the value exists from here on, whatever the branch below does
+        cand[e] = e < qn ? make_key(raw[e][0], lkm1 - raw[e][1]) : 0.0;
       }
     }
     // the queue's 13 entries through their own network; cand[13..15] stay fillers
@@ -269,17 +263,12 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < KL; i++) best[i] = cand[i];
       merge_top_desc<KL>(list, best);
-    } else {  // KL == 2 * kQCap, in place: the upper half U of the list beats its lower half M, and an element of
-      // M U cand outside that set's best kQCap cannot be among the KL best of the whole (kQCap of that set and, being
-      // below all of U, all kQCap of U are above it).  So: lower half <- best kQCap of M U cand, then one bitonic
-      // merge of the two sorted halves.
+    } else {  // KL == 2 * kQCap: the half-cleaner of a 32-wide merge only reaches the lower half of the list (the
+      // candidates, padded to the list's length with fillers, meet entries kQCap .. KL-1), in place; the list is then
+      // bitonic and holds the KL best of list U cand
       static_assert(KL == 2 * kQCap, "list lengths above the queue width are built for exactly twice that width");
-      key_t lower[kQCap];
 #pragma unroll
-      for (int i = 0; i < kQCap; i++) lower[i] = list[kQCap + i];
-      merge_top_desc<kQCap, kFill>(lower, cand);
-#pragma unroll
-      for (int i = 0; i < kQCap; i++) list[kQCap + i] = lower[kQCap - 1 - i];  // descending, then ascending: bitonic
+      for (int i = kFill; i < kQCap; i++) list[kQCap + i] = __builtin_fmax(list[kQCap + i], cand[kQCap - 1 - i]);
       bitonic_merge_desc<KL>(list);
     }
     qn = 0;
