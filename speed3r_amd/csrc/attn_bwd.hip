@@ -144,7 +144,7 @@ __device__ __forceinline__ void read_transposed(const char* half, int tr_off, ty
 #pragma unroll
     for (int dt = 0; dt < 2; dt++) {
       const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
-      const char* a8 = half + (tr_off ^ (dt * 64) ^ 64) + (jj * 16 + 8) * 128;  // rows 8 further down: chunk map ^ 4
+      const char* a8 = half + (tr_off ^ (dt * 64) ^ (k_swizzle(8) << 4)) + (jj * 16 + 8) * 128;  // rows 8 further down: chunk map ^ k_swizzle(8)
       Frag f;
       f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
       f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a8));
@@ -155,7 +155,7 @@ __device__ __forceinline__ void read_transposed(const char* half, int tr_off, ty
 template <typename E>
 __device__ __forceinline__ typename Mma<E>::V8 read_transposed_frag(const char* half, int tr_off, int jj, int dt) {
   const char* a0 = half + (tr_off ^ (dt * 64)) + (jj * 16) * 128;
-  const char* a8 = half + (tr_off ^ (dt * 64) ^ 64) + (jj * 16 + 8) * 128;
+  const char* a8 = half + (tr_off ^ (dt * 64) ^ (k_swizzle(8) << 4)) + (jj * 16 + 8) * 128;
   Frag f;
   f.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
   f.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a8));

@@ -66,14 +66,17 @@ __device__ __forceinline__ uint32_t sortable_key(float s) {
 
 constexpr int kWave = 64;
 
-// LDS layout of a tile whose rows are 128 bytes and are read as MFMA operands with ds_read_b128 (lane = row): the
-// 16-byte chunk c of row r sits at chunk position c ^ k_swizzle(r).  The LDS of this chip serves a ds_read_b128 sixteen
-// lanes at a time from 64 banks (256 bytes per clock, two rows of a tile): rows r and r + 8 share their banks, so the
-// swizzle has to tell sixteen consecutive rows apart, which (r >> 1) & 7 does together with the row's parity (the bank
-// half).  Measured on one CU with eight waves: 4.3 cycles per instruction, 8.0 with r & 7, 32 without a swizzle.
-__device__ __forceinline__ constexpr int k_swizzle(int row) {
-  return (row >> 1) & 7;
-}
+// LDS layout of a tile whose rows are 128 bytes: the 16-byte chunk c of row r sits at chunk position c ^ k_swizzle(r).
+// The LDS of this chip has 64 banks (256 bytes per clock, two rows of a tile; a row's parity picks the bank half).
+// * ds_read_b128 with lane = row (MFMA operands from rows) is served sixteen lanes at a time: rows r and r + 8 share
+//   their banks, so the map has to send row bits 1..3 to three different chunk bits.  Measured on one CU with eight
+//   waves: 4.3 cycles per instruction, 8.0 with the map r & 7, 32 without a map; a single wave does not show it.
+// * ds_read_b64_tr_b16 (operands from columns) touches, per pass, four rows r..r+3 and four chunks that differ in chunk
+//   bits 0..1: rows r and r + 2 have the same parity, so row bit 1 has to go to chunk bit 2.  (These conflicts cost
+//   bank cycles but no time in a loop that issues nothing else to the LDS: the instruction's own rate hides them.)
+// Both: row bit 1 -> chunk bit 2, row bit 2 -> chunk bit 0, row bit 3 -> chunk bit 1.  The map is linear over GF(2) in
+// the row bits, and row bit 4 and above do not enter: k_swizzle(r + 8) = k_swizzle(r) ^ k_swizzle(8) for r < 8.
+__device__ __forceinline__ constexpr int k_swizzle(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
 
 // Value held by lane ^ MASK.  Masks 1 and 2 stay inside a quad and ride on the DPP operand path of an ordinary move
 // (no LDS crossbar); masks up to 16 use the swizzle unit without an address register; larger ones the general permute.
