@@ -266,10 +266,17 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
   // key tiles of this query block
   static_assert(BLK == 64 || (BLK == 16 && !DENSE), "blocks of 64 tokens, or of 16 with an index list");
   int32_t my_idx = -1;
-  int32_t my16[4] = {-1, -1, -1, -1};  // BLK 16: entry `lane` of the lists of the wave's four query blocks
   uint64_t todo = 0;
   int ntiles;
   int dense_next = 0;
+  // BLK 16: the wave's 64 queries are four query blocks with a list each; neighbouring lists name mostly the same key
+  // blocks, so the wave walks the UNION of the four lists.  Entry n of the walk list (LDS) is a distinct key block and
+  // four count bytes (how often query block j lists it; 0: not at all, above 1: a duplicated entry, which weighs the
+  // block that often, as the forward pass does).  A tile is four entries: two per 32-key half.
+  __shared__ __attribute__((aligned(16))) int2 lds_walk[BLK == 16 ? 4 : 1][BLK == 16 ? 264 : 1];
+  int2* const walk = lds_walk[BLK == 16 ? wave : 0];
+  int n_union = 0;
+  bool dup = false;  // some list names a block more than once (wave-uniform)
   if constexpr (DENSE) {
     ntiles = (int)((Lk + 63) >> 6);
   } else if constexpr (BLK == 64) {
@@ -279,6 +286,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     ntiles = __popcll(todo);
   } else {
     const int64_t nqb16 = (Lq + 15) >> 4;
+    int32_t my16[4] = {-1, -1, -1, -1};  // entry `lane` of the four lists
 #pragma unroll
     for (int s = 0; s < 4; s++) {
       const int64_t qb16 = (int64_t)qb * 4 + s;
@@ -287,7 +295,50 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
         my16[s] = (v >= 0 && (int64_t)v * 16 < Lk) ? v : -1;
       }
     }
-    ntiles = p.K;  // entry t of all four lists makes tile t; entries that are skipped get P = 0
+    // Distinct blocks and their counts through a hash table in LDS (512 slots in this wave's first K buffer, which no
+    // transfer touches before the list is complete): every lane inserts its entry of list j with a compare-and-swap on
+    // the key (linear probing; at most 4 x 64 distinct blocks) and adds 1 << 8j to the slot's count; the occupied
+    // slots are then compacted into the list, eight slots per lane, positions from ballots.
+    int32_t* const hkey = reinterpret_cast<int32_t*>(k_buf[0]);          // [512]
+    uint32_t* const hcnt = reinterpret_cast<uint32_t*>(k_buf[0] + 2048);  // [512]
+    reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
+    reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
+    reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
+    reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int32_t e = my16[j];
+      bool active = e >= 0;
+      uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
+      while (active) {
+        const int32_t old = atomicCAS(hkey + slot, -1, e);
+        if (old == -1 || old == e) {
+          atomicAdd(hcnt + slot, 1u << (8 * j));
+          active = false;
+        } else {
+          slot = (slot + 1) & 511u;
+        }
+      }
+    }
+    const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
+    const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
+    const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+    const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    uint32_t pos = 0;  // occupied slots of the lanes below
+    uint32_t cnt_bits = 0;
+#pragma unroll
+    for (int s8 = 0; s8 < 8; s8++) {
+      const uint64_t m = __ballot(ks8[s8] >= 0);
+      pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
+      n_union += __popcll(m);
+      cnt_bits |= (uint32_t)cs8[s8];
+    }
+#pragma unroll
+    for (int s8 = 0; s8 < 8; s8++)
+      if (ks8[s8] >= 0) walk[pos++] = make_int2(ks8[s8], cs8[s8]);
+    dup = __any((cnt_bits & 0xfefefefeu) != 0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the table is read and the list written before the first transfer
+    ntiles = (n_union + 3) >> 2;
   }
   auto pop = [&]() -> int64_t {  // start row of the next tile, BLK 16: its list position (callers pop exactly ntiles times)
     if constexpr (DENSE) {
@@ -300,11 +351,16 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       return (int64_t)(dense_next++);
     }
   };
-  // BLK 16: first key row and number of valid rows (0: skipped) of block `s` of tile t
-  auto sub_block = [&](int64_t t, int s, int64_t& start, int& nv) {
-    const int32_t v = __builtin_amdgcn_readlane(my16[s], (int)t);
-    start = v >= 0 ? (int64_t)v * 16 : 0;
-    nv = v >= 0 ? (int)(Lk - start < 16 ? Lk - start : 16) : 0;
+  // BLK 16: first key row, number of valid rows and the four count bytes of entry `s` (0..3) of tile t of the walk
+  // list (past the list's end: row 0, no counts)
+  auto sub_block = [&](int64_t t, int s, int64_t& start, int& nv, uint32_t& counts) {
+    const int e = 4 * (int)t + s;
+    int2 v = make_int2(-1, 0);
+    if (e < n_union) v = walk[e];
+    const int32_t blk = __builtin_amdgcn_readfirstlane(v.x);
+    counts = (uint32_t)__builtin_amdgcn_readfirstlane(v.y);
+    start = blk >= 0 ? (int64_t)blk * 16 : 0;
+    nv = blk >= 0 ? (int)(Lk - start < 16 ? Lk - start : 16) : 0;
   };
 
   const float scale = p.scale;
@@ -321,8 +377,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     } else {
       int64_t sa, sb;
       int na, nb;
-      sub_block(start, 2 * HF, sa, na);
-      sub_block(start, 2 * HF + 1, sb, nb);
+      uint32_t ca, cb;
+      sub_block(start, 2 * HF, sa, na, ca);
+      sub_block(start, 2 * HF + 1, sb, nb, cb);
       const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
       dma_rows16<E, true>(kp + sa * p.skn, kp + sb * p.skn, krow, la, lb, k_buf[buf], lane);
       dma_rows16<E, false>(vp + sa * p.svn, vp + sb * p.svn, vrow, la, lb, v_buf[buf], lane);
@@ -331,22 +388,21 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
   auto compute = [&](int64_t start, auto hf, int buf) {
     constexpr int HF = decltype(hf)::value;
     int nvalid = 64;
-    int nv_mine = 16;  // BLK 16: valid keys of the block that this lane's query attends to in this half
+    int na = 16, nb = 16;      // BLK 16: valid keys of the half's two blocks A (rows 0..15) and B (16..31)
+    uint32_t ca = 0, cb = 0;   // and how often each of the four query blocks lists them
     if constexpr (BLK == 64) {
       nvalid = (int)(Lk - start < 64 ? Lk - start : 64);
     } else {
       int64_t sa, sb;
-      int na, nb;
-      sub_block(start, 2 * HF, sa, na);
-      sub_block(start, 2 * HF + 1, sb, nb);
-      nv_mine = (c >> 4) ? nb : na;
+      sub_block(start, 2 * HF, sa, na, ca);
+      sub_block(start, 2 * HF + 1, sb, nb, cb);
     }
     const bool ragged = nvalid < 64;
     V8 ak[4], av[4];
     read_rows<E, true>(k_buf[buf], c, hh, ak);
     read_rows<E, false>(v_buf[buf], c, hh, av);
     V8 ds[2][2];  // dS^T as B operand [qt][jj]
-    constexpr int QT0 = BLK == 64 ? 0 : HF, QT1 = BLK == 64 ? 2 : HF + 1;  // BLK 16: key half h meets query half h only
+    constexpr int QT0 = 0, QT1 = 2;
 #pragma unroll
     for (int qt = QT0; qt < QT1; qt++) {
       f32x16 st, dp;
@@ -364,10 +420,19 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
           for (int r = 0; r < 16; r++)
             if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) st[r] = 0.f;
         }
-      } else {  // registers 0..7 are keys of block A, 8..15 of block B; this lane's query belongs to one of them
+      } else {  // registers 0..7 are keys of block A, 8..15 of block B; this lane's query block lists each 0, 1 or more times
+        const int sh = 8 * (2 * qt + (c >> 4));
+        const uint32_t wa = (ca >> sh) & 0xffu, wb = (cb >> sh) & 0xffu;
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-          if ((r >> 3) != (c >> 4) || 4 * hh + 8 * ((r >> 2) & 1) + (r & 3) >= nv_mine) st[r] = 0.f;
+        for (int r = 0; r < 16; r++) {
+          const bool on = (r < 8 ? wa : wb) != 0 && 4 * hh + 8 * ((r >> 2) & 1) + (r & 3) < (r < 8 ? na : nb);
+          st[r] = on ? st[r] : 0.f;
+        }
+        if (dup) {
+          const float fa = (float)wa, fb = (float)wb;
+#pragma unroll
+          for (int r = 0; r < 16; r++) st[r] *= r < 8 ? fa : fb;
+        }
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[qt][r >> 3][r & 7] = (E)(st[r] * fmaf(dp[r], scale, -dlts[qt]));  // scale * P * (dP - delta)
