@@ -162,6 +162,51 @@ __device__ __forceinline__ typename Mma<E>::V8 read_transposed_frag(const char* 
   return as_v8<E>(f);
 }
 
+// The same reads written by hand and waited for by the caller (lds_wait): the compiler neither sees an LDS access nor
+// adds a wait of its own.  A compiler-visible LDS read that follows direct transfers into LDS makes it wait for every
+// transfer that it cannot tell apart from the buffer being read, here also those of the NEXT half tile, which have just
+// been issued.  The values must not be touched before lds_wait.
+template <typename E>
+__device__ __forceinline__ void read_rows_async(const char* half, int c, int hh, u32x4 (&dst)[4]) {
+  // one address register: row and the chunk of k-step 0; the k-step flips chunk bits 1..2 (tiles are 1 KB aligned).
+  // The empty asm keeps the four addresses from being computed ahead of the loop and held in registers.
+  uint32_t a0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half + (uint32_t)(c * 128 + ((hh ^ k_swizzle(c)) << 4));
+  asm volatile("" : "+v"(a0));
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) asm volatile("ds_read_b128 %0, %1" : "=v"(dst[ks]) : "v"(a0 ^ (uint32_t)(ks << 5)));
+}
+template <typename E>
+__device__ __forceinline__ void read_transposed_async(const char* half, int tr_off, u32x2 (&dst)[2][2][2]) {  // [jj][dt][rows 0-7 | 8-15]
+  uint32_t t0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half + (uint32_t)tr_off;
+  asm volatile("" : "+v"(t0));
+#pragma unroll
+  for (int dt = 0; dt < 2; dt++) {
+    const uint32_t a0 = t0 ^ (uint32_t)(dt * 64);
+    const uint32_t a8 = a0 ^ (uint32_t)(k_swizzle(8) << 4);  // rows 8 further down: chunk map ^ k_swizzle(8)
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst[0][dt][0]) : "v"(a0));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:1024" : "=v"(dst[0][dt][1]) : "v"(a8));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(dst[1][dt][0]) : "v"(a0));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:3072" : "=v"(dst[1][dt][1]) : "v"(a8));
+  }
+}
+__device__ __forceinline__ void lds_wait(u32x4 (&a)[4], u32x4 (&b)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+}
+__device__ __forceinline__ void lds_wait(u32x2 (&a)[2][2][2]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(a[0][0][0]), "+v"(a[0][0][1]), "+v"(a[0][1][0]), "+v"(a[0][1][1]), "+v"(a[1][0][0]), "+v"(a[1][0][1]), "+v"(a[1][1][0]), "+v"(a[1][1][1]));
+}
+template <typename E> __device__ __forceinline__ typename Mma<E>::V8 frag_of(u32x4 w) {
+  Frag f;
+  f.u = make_uint4(w[0], w[1], w[2], w[3]);
+  return as_v8<E>(f);
+}
+template <typename E> __device__ __forceinline__ typename Mma<E>::V8 frag_of(u32x2 lo, u32x2 hi) {
+  Frag f;
+  f.u = make_uint4(lo[0], lo[1], hi[0], hi[1]);
+  return as_v8<E>(f);
+}
+
 __device__ __forceinline__ int tr_offset(int lane) {
   const int hh = lane >> 5;
   const int i16 = lane & 15;
@@ -355,10 +400,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
   // list (past the list's end: row 0, no counts)
   auto sub_block = [&](int64_t t, int s, int64_t& start, int& nv, uint32_t& counts) {
     const int e = 4 * (int)t + s;
-    int2 v = make_int2(-1, 0);
-    if (e < n_union) v = walk[e];
-    const int32_t blk = __builtin_amdgcn_readfirstlane(v.x);
-    counts = (uint32_t)__builtin_amdgcn_readfirstlane(v.y);
+    u32x2 v = {0xffffffffu, 0u};
+    if (e < n_union) {  // (wave-uniform) a hand-written read, like the fragments'
+      const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)reinterpret_cast<const char*>(walk + e);
+      asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a));
+    }
+    const int32_t blk = __builtin_amdgcn_readfirstlane((int32_t)v[0]);
+    counts = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v[1]);
     start = blk >= 0 ? (int64_t)blk * 16 : 0;
     nv = blk >= 0 ? (int)(Lk - start < 16 ? Lk - start : 16) : 0;
   };
@@ -399,8 +447,17 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     }
     const bool ragged = nvalid < 64;
     V8 ak[4], av[4];
-    read_rows<E, true>(k_buf[buf], c, hh, ak);
-    read_rows<E, false>(v_buf[buf], c, hh, av);
+    {
+      u32x4 kw[4], vw[4];
+      read_rows_async<E>(k_buf[buf], c, hh, kw);
+      read_rows_async<E>(v_buf[buf], c, hh, vw);
+      lds_wait(kw, vw);
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        ak[ks] = frag_of<E>(kw[ks]);
+        av[ks] = frag_of<E>(vw[ks]);
+      }
+    }
     V8 ds[2][2];  // dS^T as B operand [qt][jj]
     constexpr int QT0 = 0, QT1 = 2;
 #pragma unroll
@@ -438,7 +495,15 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       for (int r = 0; r < 16; r++) ds[qt][r >> 3][r & 7] = (E)(st[r] * fmaf(dp[r], scale, -dlts[qt]));  // scale * P * (dP - delta)
     }
     V8 kt[2][2];
-    read_transposed<E>(k_buf[buf], tr_off, kt);
+    {
+      u32x2 tw[2][2][2];
+      read_transposed_async<E>(k_buf[buf], tr_off, tw);
+      lds_wait(tw);
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) kt[jj][dt] = frag_of<E>(tw[jj][dt][0], tw[jj][dt][1]);
+    }
 #pragma unroll
     for (int jj = 0; jj < 2; jj++)
 #pragma unroll
