@@ -140,10 +140,19 @@ template <int OFF> __device__ __forceinline__ u32x4 lds_read16_async(uint32_t ad
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
 }
-template <int OFF> __device__ __forceinline__ u32x2 lds_read8_async(uint32_t addr) {
-  u32x2 v;
-  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
-  return v;
+// The 13 slots of a lane's queue (64 x 8 bytes apart) in one statement, reads and wait together: between a hand-written
+// read and its wait the compiler must not get a chance to move or spill a register whose value has not arrived.
+__device__ __forceinline__ void lds_read_queue13(uint32_t addr, u32x2 (&r)[13]) {
+  asm volatile(
+      "ds_read_b64 %0, %13\n\tds_read_b64 %1, %13 offset:512\n\tds_read_b64 %2, %13 offset:1024\n\t"
+      "ds_read_b64 %3, %13 offset:1536\n\tds_read_b64 %4, %13 offset:2048\n\tds_read_b64 %5, %13 offset:2560\n\t"
+      "ds_read_b64 %6, %13 offset:3072\n\tds_read_b64 %7, %13 offset:3584\n\tds_read_b64 %8, %13 offset:4096\n\t"
+      "ds_read_b64 %9, %13 offset:4608\n\tds_read_b64 %10, %13 offset:5120\n\tds_read_b64 %11, %13 offset:5632\n\t"
+      "ds_read_b64 %12, %13 offset:6144\n\ts_waitcnt lgkmcnt(0)"
+      : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]), "=&v"(r[4]), "=&v"(r[5]), "=&v"(r[6]), "=&v"(r[7]), "=&v"(r[8]),
+        "=&v"(r[9]), "=&v"(r[10]), "=&v"(r[11]), "=&v"(r[12])
+      : "v"(addr)
+      : "memory");
 }
 __device__ __forceinline__ void lds_reads_done(u32x4 (&a)[2][4]) {
   asm volatile("s_waitcnt lgkmcnt(0)"
@@ -236,19 +245,16 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
     // All queue slots are fetched at once and waited for once (hand-written reads: left to the compiler, each read
     // lands inside the `e < qn` branch of its entry with a wait of its own, thirteen LDS round trips in a row;
     // top-16 at 4 164 keys 0.148 -> 0.140 ms).
-    u32x2 raw[kQSlots > 1 ? kQSlots - 1 : 1];  // (the attention instance has no queue and never folds)
-    {
-      const uint32_t qaddr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(qlane);
-#pragma unroll
-      for (int e = 0; e < kQSlots - 1; e++) raw[e] = lds_read8_async<0>(qaddr + e * 64 * 8);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    u32x2 raw[13];
+    if constexpr (FUSED) {  // (the attention instance has no queue and never folds)
+      static_assert(!FUSED || kQSlots - 1 == 13, "the fold reads 13 queue slots");
+      lds_read_queue13((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(qlane), raw);
     }
     key_t cand[kQCap];
 #pragma unroll
     for (int e = 0; e < kQCap; e++) {
       cand[e] = 0;
       if (e < kQSlots - 1) {
-        asm volatile("" : "+v"(raw[e]));  // the value exists from here on, whatever the branch below does
         cand[e] = e < qn ? make_key(raw[e][0], lkm1 - raw[e][1]) : 0.0;
       }
     }
