@@ -162,39 +162,41 @@ __device__ __forceinline__ typename Mma<E>::V8 read_transposed_frag(const char* 
   return as_v8<E>(f);
 }
 
-// The same reads written by hand and waited for by the caller (lds_wait): the compiler neither sees an LDS access nor
-// adds a wait of its own.  A compiler-visible LDS read that follows direct transfers into LDS makes it wait for every
-// transfer that it cannot tell apart from the buffer being read, here also those of the NEXT half tile, which have just
-// been issued.  The values must not be touched before lds_wait.
-template <typename E>
-__device__ __forceinline__ void read_rows_async(const char* half, int c, int hh, u32x4 (&dst)[4]) {
-  // one address register: row and the chunk of k-step 0; the k-step flips chunk bits 1..2 (tiles are 1 KB aligned).
-  // The empty asm keeps the four addresses from being computed ahead of the loop and held in registers.
-  uint32_t a0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half + (uint32_t)(c * 128 + ((hh ^ k_swizzle(c)) << 4));
-  asm volatile("" : "+v"(a0));
-#pragma unroll
-  for (int ks = 0; ks < 4; ks++) asm volatile("ds_read_b128 %0, %1" : "=v"(dst[ks]) : "v"(a0 ^ (uint32_t)(ks << 5)));
+// The same reads written by hand, each group one asm statement that ends with its own wait: the compiler neither sees an
+// LDS access nor adds a wait of its own, and no register of an outstanding read is left to the register allocator.  A
+// compiler-visible LDS read that follows direct transfers into LDS makes the compiler wait for every transfer that it
+// cannot tell apart from the buffer being read, here also those of the NEXT half tile, which have just been issued.
+// Row fragments of two half tiles (K and V, or Q and dO): lane = row c, k-step ks: head_dim chunk 2ks + hh.
+__device__ __forceinline__ void read_rows2_sync(const char* half_a, const char* half_b, int c, int hh, u32x4 (&a)[4], u32x4 (&b)[4]) {
+  // one address per tile: row and the chunk of k-step 0; the k-step flips chunk bits 1..2 (tiles are 1 KB aligned).
+  // The empty asm keeps the eight addresses from being computed ahead of the loop and held in registers.
+  const uint32_t off = (uint32_t)(c * 128 + ((hh ^ k_swizzle(c)) << 4));
+  uint32_t a0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half_a + off;
+  uint32_t b0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half_b + off;
+  asm volatile("" : "+v"(a0), "+v"(b0));
+  asm volatile(
+      "ds_read_b128 %0, %8\n\tds_read_b128 %1, %9\n\tds_read_b128 %2, %10\n\tds_read_b128 %3, %11\n\t"
+      "ds_read_b128 %4, %12\n\tds_read_b128 %5, %13\n\tds_read_b128 %6, %14\n\tds_read_b128 %7, %15\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3]), "=&v"(b[0]), "=&v"(b[1]), "=&v"(b[2]), "=&v"(b[3])
+      : "v"(a0), "v"(a0 ^ 32u), "v"(a0 ^ 64u), "v"(a0 ^ 96u), "v"(b0), "v"(b0 ^ 32u), "v"(b0 ^ 64u), "v"(b0 ^ 96u)
+      : "memory");
 }
-template <typename E>
-__device__ __forceinline__ void read_transposed_async(const char* half, int tr_off, u32x2 (&dst)[2][2][2]) {  // [jj][dt][rows 0-7 | 8-15]
+// Transposed fragments of one half tile: dst[jj][dt][rows 0-7 | 8-15 of the 16-row group jj].
+__device__ __forceinline__ void read_transposed_sync(const char* half, int tr_off, u32x2 (&dst)[2][2][2]) {
   uint32_t t0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)half + (uint32_t)tr_off;
   asm volatile("" : "+v"(t0));
-#pragma unroll
-  for (int dt = 0; dt < 2; dt++) {
-    const uint32_t a0 = t0 ^ (uint32_t)(dt * 64);
-    const uint32_t a8 = a0 ^ (uint32_t)(k_swizzle(8) << 4);  // rows 8 further down: chunk map ^ k_swizzle(8)
-    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst[0][dt][0]) : "v"(a0));
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:1024" : "=v"(dst[0][dt][1]) : "v"(a8));
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(dst[1][dt][0]) : "v"(a0));
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:3072" : "=v"(dst[1][dt][1]) : "v"(a8));
-  }
-}
-__device__ __forceinline__ void lds_wait(u32x4 (&a)[4], u32x4 (&b)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-}
-__device__ __forceinline__ void lds_wait(u32x2 (&a)[2][2][2]) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(a[0][0][0]), "+v"(a[0][0][1]), "+v"(a[0][1][0]), "+v"(a[0][1][1]), "+v"(a[1][0][0]), "+v"(a[1][0][1]), "+v"(a[1][1][0]), "+v"(a[1][1][1]));
+  const uint32_t t8 = t0 ^ (uint32_t)(k_swizzle(8) << 4);  // rows 8 further down: chunk map ^ k_swizzle(8)
+  asm volatile(
+      "ds_read_b64_tr_b16 %0, %8\n\tds_read_b64_tr_b16 %1, %10 offset:1024\n\t"
+      "ds_read_b64_tr_b16 %2, %9\n\tds_read_b64_tr_b16 %3, %11 offset:1024\n\t"
+      "ds_read_b64_tr_b16 %4, %8 offset:2048\n\tds_read_b64_tr_b16 %5, %10 offset:3072\n\t"
+      "ds_read_b64_tr_b16 %6, %9 offset:2048\n\tds_read_b64_tr_b16 %7, %11 offset:3072\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(dst[0][0][0]), "=&v"(dst[0][0][1]), "=&v"(dst[0][1][0]), "=&v"(dst[0][1][1]), "=&v"(dst[1][0][0]), "=&v"(dst[1][0][1]),
+        "=&v"(dst[1][1][0]), "=&v"(dst[1][1][1])
+      : "v"(t0), "v"(t0 ^ 64u), "v"(t8), "v"(t8 ^ 64u)
+      : "memory");
 }
 template <typename E> __device__ __forceinline__ typename Mma<E>::V8 frag_of(u32x4 w) {
   Frag f;
@@ -449,9 +451,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     V8 ak[4], av[4];
     {
       u32x4 kw[4], vw[4];
-      read_rows_async<E>(k_buf[buf], c, hh, kw);
-      read_rows_async<E>(v_buf[buf], c, hh, vw);
-      lds_wait(kw, vw);
+      read_rows2_sync(k_buf[buf], v_buf[buf], c, hh, kw, vw);
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) {
         ak[ks] = frag_of<E>(kw[ks]);
@@ -497,8 +497,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
     V8 kt[2][2];
     {
       u32x2 tw[2][2][2];
-      read_transposed_async<E>(k_buf[buf], tr_off, tw);
-      lds_wait(tw);
+      read_transposed_sync(k_buf[buf], tr_off, tw);
 #pragma unroll
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
