@@ -133,12 +133,18 @@ template <> struct TopkCfg<0> {
   static constexpr int kRing = 2;
 };
 
-// LDS read whose completion the caller waits for itself (lds_reads_done): the compiler neither knows that it reads
-// LDS nor when it lands, so it adds no wait for transfers into other LDS buffers that are still in flight.
-template <int OFF> __device__ __forceinline__ u32x4 lds_read16_async(uint32_t addr) {
-  u32x4 v;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
-  return v;
+// The eight K fragments of a 64-key tile, rows c (f[0]) and c + 32 (f[1]), k-steps 0..3 (chunk bits 1..2 of the address),
+// read by hand: the compiler neither knows that this reads LDS nor when it lands, so it adds no wait for transfers into
+// other LDS buffers that are still in flight.  Reads and wait are one statement: between a hand-written read and its
+// wait the compiler must not get a chance to move or spill a register whose value has not arrived.
+__device__ __forceinline__ void lds_read_kfrags(uint32_t kb, u32x4 (&f)[2][4]) {
+  asm volatile(
+      "ds_read_b128 %0, %8\n\tds_read_b128 %4, %8 offset:4096\n\tds_read_b128 %1, %9\n\tds_read_b128 %5, %9 offset:4096\n\t"
+      "ds_read_b128 %2, %10\n\tds_read_b128 %6, %10 offset:4096\n\tds_read_b128 %3, %11\n\tds_read_b128 %7, %11 offset:4096\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(f[0][0]), "=&v"(f[0][1]), "=&v"(f[0][2]), "=&v"(f[0][3]), "=&v"(f[1][0]), "=&v"(f[1][1]), "=&v"(f[1][2]), "=&v"(f[1][3])
+      : "v"(kb), "v"(kb ^ 32u), "v"(kb ^ 64u), "v"(kb ^ 96u)
+      : "memory");
 }
 // The 13 slots of a lane's queue (64 x 8 bytes apart) in one statement, reads and wait together: between a hand-written
 // read and its wait the compiler must not get a chance to move or spill a register whose value has not arrived.
@@ -153,10 +159,6 @@ __device__ __forceinline__ void lds_read_queue13(uint32_t addr, u32x2 (&r)[13]) 
         "=&v"(r[9]), "=&v"(r[10]), "=&v"(r[11]), "=&v"(r[12])
       : "v"(addr)
       : "memory");
-}
-__device__ __forceinline__ void lds_reads_done(u32x4 (&a)[2][4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]), "+v"(a[1][0]), "+v"(a[1][1]), "+v"(a[1][2]), "+v"(a[1][3]));
 }
 
 template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */>
@@ -469,12 +471,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
           const bool partial = start + 64 > Lk;
           u32x4 kf[2][4];
           const uint32_t kb = kr_off + (uint32_t)buf * (kTile * (uint32_t)sizeof(E));
-#pragma unroll
-          for (int ks = 0; ks < 4; ks++) {
-            kf[0][ks] = lds_read16_async<0>(kb ^ (ks << 5));
-            kf[1][ks] = lds_read16_async<32 * 128>(kb ^ (ks << 5));
-          }
-          lds_reads_done(kf);
+          lds_read_kfrags(kb, kf);
           f32x16 st[2];
 #pragma unroll
           for (int kt = 0; kt < 2; kt++) {
