@@ -2,11 +2,11 @@
 // dense non-causal flash attention over the pooled tokens, plus the exact top-k block
 // selection, either fused into the same pass or from a score matrix written to HBM.
 //
-// A 256-thread workgroup owns 128 query rows of one head, 32 per wavefront, and walks all key
+// A workgroup of four wavefronts (the top-k-only kernel also: two) owns 32 query rows of one head per wavefront and walks all key
 // tiles of 64 pooled tokens.  K and V tiles are staged once per workgroup in LDS (global ->
 // registers two tiles ahead -> LDS one tile ahead, two LDS buffers, one barrier per tile) and
 // shared by the four waves.  Rows are 128 bytes without padding; 16-byte chunks are stored
-// XOR-swizzled (K: chunk ^ ((row >> 1) & 7) for the 16-byte operand reads, V: halves swapped on rows
+// XOR-swizzled (K: chunk ^ k_swizzle(row) for the 16-byte operand reads, V: halves swapped on rows
 // 2,3 mod 4 for the transposed reads) so that LDS reads are bank-conflict free.
 // Per wave and tile: S^T = K Q^T with v_mfma_f32_32x32x16 (one query per lane and its partner
 // lane ^ 32, 32 of the tile's 64 keys in each lane's registers), base-2 online softmax in
@@ -161,16 +161,23 @@ __device__ __forceinline__ void lds_read_queue13(uint32_t addr, u32x2 (&r)[13]) 
       : "memory");
 }
 
-template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */>
+// WAVES: wavefronts (of 32 query rows) per workgroup.  The top-k-only kernel also comes with two: its waves meet at a
+// barrier per tile, so whatever one wave does beyond the common path (a fold of its queues) holds up its whole
+// workgroup; with few workgroups (one round, nothing else on the SIMD to fill the gap) pairs lose less than quads.
+// Two waves per workgroup double the K tile transfers per query row and use a ring of two tiles (30 KB of LDS with the
+// queues, five workgroups per CU).
+template <typename E, int KTOP /* 0: attention (+ scores); > 0: top-k only */, int WAVES>
 __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(AttnParams p) {
   typedef typename Mma<E>::V8 V8;
   constexpr bool FUSED = KTOP > 0;
+  static_assert(WAVES == 4 || (WAVES == 2 && FUSED), "two waves per workgroup: top-k-only kernel");
   constexpr int KL = FUSED ? KTOP : 1;  // list length per lane
   constexpr int kQSlots = TopkCfg<KTOP>::kQSlots;
-  constexpr int NB = TopkCfg<KTOP>::kRing;
+  constexpr int NB = WAVES == 2 ? 2 : TopkCfg<KTOP>::kRing;
+  constexpr int NI = 8 / WAVES;  // transfer instructions (8 rows each) per wave and tile
   __shared__ __attribute__((aligned(1024))) E Ks[NB][kTile];
   __shared__ __attribute__((aligned(1024))) E Vs[FUSED ? 1 : 2][FUSED ? 8 : kTile];  // the top-k-only kernel stages K tiles alone
-  __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? 4 : 1][kQSlots][64];
+  __shared__ __attribute__((aligned(16))) uint2 queue[FUSED ? WAVES : 1][kQSlots][64];
   __shared__ __attribute__((aligned(16))) float sstage[FUSED ? 1 : 4][FUSED ? 4 : 32 * 64];  // score-store staging (unfused launches)
 
   const int tid = threadIdx.x;
@@ -181,7 +188,7 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
   const int b = blockIdx.y / p.H;
   const int h = blockIdx.y - b * p.H;
   const int64_t Lq = p.Lq, Lk = p.Lk;
-  const int64_t q0 = (int64_t)blockIdx.x * 128 + wave * 32;
+  const int64_t q0 = (int64_t)blockIdx.x * (32 * WAVES) + wave * 32;
 
   const E* qp = (const E*)p.q + (int64_t)b * p.sqb + (int64_t)h * p.sqh;
   const E* kp = (const E*)p.k + (int64_t)b * p.skb + (int64_t)h * p.skh;
@@ -426,31 +433,36 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
   if constexpr (FUSED) {
     // One sweep over the key tiles: S^T by MFMA, then either the group maxima (first sweep) or the candidate filter
     // (second sweep).  K tiles go global -> LDS by direct transfers into a ring of NB buffers, NB - 1 tiles ahead of
-    // the tile being read; wave w moves rows 16w .. 16w+15 of a tile (two instructions of 8 rows).  LDS chunk
+    // the tile being read; wave w moves rows 8 NI w .. 8 NI (w + 1) - 1 of a tile (NI instructions of 8 rows).  LDS chunk
     // (row, c') holds head_dim chunk c' ^ k_swizzle(row).  Rows beyond Lk re-read the last row (they are masked).
     const uint32_t krow_bytes = (uint32_t)p.skn * (uint32_t)sizeof(E);
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // the LDS destination of a transfer is a scalar (M0)
-    const int dl_row = wave_u * 16 + (lane >> 3);
+    const int dl_row = wave_u * (8 * NI) + (lane >> 3);
+    // (the chunk map repeats every 16 rows: instructions of equal parity share it)
     const uint32_t dl_chunk[2] = {(uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16), (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
-    const uint32_t dl_off[2] = {(uint32_t)dl_row * krow_bytes + dl_chunk[0], (uint32_t)(dl_row + 8) * krow_bytes + dl_chunk[1]};
+    uint32_t dl_off[4] = {0, 0, 0, 0};  // NI of them are used
+#pragma unroll
+    for (int i = 0; i < NI; i++) dl_off[i] = (uint32_t)(dl_row + 8 * i) * krow_bytes + dl_chunk[i & 1];
     auto dma_tile = [&](int t, int buf) {  // tiles past the end repeat the last one (never read)
       const int tt = t < ntiles ? t : ntiles - 1;
       const int64_t start = (int64_t)tt * 64;
       const int rem = (int)(Lk - 1 - start);
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + start * p.skn), 0, 0x7fffffff, 0x00020000);
-      char* dst = reinterpret_cast<char*>(&Ks[buf][0]) + wave_u * 2048;
-      uint32_t off[2] = {dl_off[0], dl_off[1]};  // the per-lane offsets of a full tile never change
+      char* dst = reinterpret_cast<char*>(&Ks[buf][0]) + wave_u * (NI * 1024);
+      uint32_t off[4] = {0, 0, 0, 0};  // the per-lane offsets of a full tile never change
+#pragma unroll
+      for (int i = 0; i < NI; i++) off[i] = dl_off[i];
       if (__builtin_expect(rem < 63, 0)) {       // ragged last tile: rows beyond the end re-read the last row
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < NI; i++) {
           int r = dl_row + 8 * i;
           r = r < rem ? r : rem;
-          off[i] = (uint32_t)r * krow_bytes + dl_chunk[i];
+          off[i] = (uint32_t)r * krow_bytes + dl_chunk[i & 1];
           asm volatile("" : "+v"(off[i]));       // stays inside this branch
         }
       }
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < NI; i++)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, off[i], 0, 0, 0);
     };
     const uint32_t lds_k = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)reinterpret_cast<char*>(&Ks[0][0]);
@@ -462,8 +474,8 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       int buf = 0, fill = NB - 1;  // ring positions of step i's tile and of step i + NB - 1's
       for (int i = 0; i < nsteps; i++) {
         const int t = i * stride;
-        // this wave's share of tile t has landed (transfers complete in order, two per tile, NB - 2 tiles younger) ...
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NB - 2)));
+        // this wave's share of tile t has landed (transfers complete in order, NI per tile, NB - 2 tiles younger) ...
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (NI * (NB - 2)));
         __builtin_amdgcn_s_barrier();  // ... and everybody's; all waves are done with tile t - 1, whose buffer is refilled now
         dma_tile((i + NB - 1) * stride, fill);
         {
@@ -616,22 +628,39 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
 
 template <typename E>
 static int launch_e(const AttnParams& p, bool fused, hipStream_t st) {
-  const int64_t nqg = (p.Lq + 127) / 128;
-  if (nqg > 0x7fffffffLL || (int64_t)p.B * p.H > 65535) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: grid too large");
-  dim3 grid((unsigned)nqg, (unsigned)(p.B * p.H)), blk(256);
+  if ((int64_t)p.B * p.H > 65535) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: grid too large");
   if (!fused) {
-    hipLaunchKernelGGL((compressed_mfma_kernel<E, 0>), grid, blk, 0, st, p);
-  } else {
-    switch (p.K) {
-      case 1: hipLaunchKernelGGL((compressed_mfma_kernel<E, 1>), grid, blk, 0, st, p); break;
-      case 2: hipLaunchKernelGGL((compressed_mfma_kernel<E, 2>), grid, blk, 0, st, p); break;
-      case 4: hipLaunchKernelGGL((compressed_mfma_kernel<E, 4>), grid, blk, 0, st, p); break;
-      case 8: hipLaunchKernelGGL((compressed_mfma_kernel<E, 8>), grid, blk, 0, st, p); break;
-      case 16: hipLaunchKernelGGL((compressed_mfma_kernel<E, 16>), grid, blk, 0, st, p); break;
-      case 32: hipLaunchKernelGGL((compressed_mfma_kernel<E, 32>), grid, blk, 0, st, p); break;
-      default: return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}");
-    }
+    const int64_t nqg = (p.Lq + 127) / 128;
+    if (nqg > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: grid too large");
+    dim3 grid((unsigned)nqg, (unsigned)(p.B * p.H)), blk(256);
+    hipLaunchKernelGGL((compressed_mfma_kernel<E, 0, 4>), grid, blk, 0, st, p);
+    return check_launch("compressed_mfma_kernel");
   }
+  // Workgroups of two waves where those of four would leave the chip one round with idle slots (more than one and a
+  // half per CU, at most three) and the pairs still fit it at once (five per CU): 4 164 pooled tokens x 16 heads are 528
+  // quads or 1056 pairs, top-16 0.125 -> 0.115 ms, top-32 0.200 -> 0.175 ms.  With more rows the quads' shared tiles win
+  // (16 266 tokens: pairs +7 %), with fewer the transfers' latency does (1 041 tokens: pairs +2 .. 15 %).
+  const int64_t pairs = ((p.Lq + 63) / 64) * (int64_t)p.B * p.H;
+  const bool two = pairs > 3 * 256 && pairs <= 5 * 256;
+  const int waves = two ? 2 : 4;
+  const int64_t nqg = (p.Lq + 32 * waves - 1) / (32 * waves);
+  if (nqg > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: grid too large");
+  dim3 grid((unsigned)nqg, (unsigned)(p.B * p.H)), blk(64 * waves);
+#define S3R_LAUNCH_TOPK(K)                                                              \
+  case K:                                                                               \
+    if (two) hipLaunchKernelGGL((compressed_mfma_kernel<E, K, 2>), grid, blk, 0, st, p); \
+    else hipLaunchKernelGGL((compressed_mfma_kernel<E, K, 4>), grid, blk, 0, st, p);     \
+    break;
+  switch (p.K) {
+    S3R_LAUNCH_TOPK(1)
+    S3R_LAUNCH_TOPK(2)
+    S3R_LAUNCH_TOPK(4)
+    S3R_LAUNCH_TOPK(8)
+    S3R_LAUNCH_TOPK(16)
+    S3R_LAUNCH_TOPK(32)
+    default: return fail(S3R_ERR_UNSUPPORTED, "s3r_compressed_attn_topk: fused selection is built for top-k in {1,2,4,8,16,32}");
+  }
+#undef S3R_LAUNCH_TOPK
   return check_launch("compressed_mfma_kernel");
 }
 

@@ -163,6 +163,27 @@ def test_fused_selection_equals_selection_from_stored_scores(dtype, k, lq, lk):
     assert max_abs(o_f, o_m.float()) <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("k", [1, 8, 16, 32])
+@pytest.mark.parametrize("h,lq,lk", [(26, 2000, 300), (16, 4164, 1041), (13, 4100, 65)])
+def test_fused_selection_in_two_wave_workgroups(dtype, k, h, lq, lk):
+    """Between 768 and 1280 (64-row block, head) pairs the index kernel runs workgroups of two waves (a ring of two K
+    tiles, four transfer instructions per wave and tile): the same bit-exact agreement with the oracle's order on the
+    stored scores, ties included, ragged last query block and ragged last key tile."""
+    pairs = -(-lq // 64) * h
+    assert 768 < pairs <= 1280
+    q = _randn((1, h, lq, 64), lq + k, dtype, 0.5).to(DEV)
+    kk = _randn((1, h, lk, 64), lk + 1, dtype, 0.5)
+    kk[:, :, lk // 2:] = kk[:, :, :lk - lk // 2]          # duplicated keys: exact score ties, lowest column must win
+    kk = kk.to(DEV)
+    _, idx_f = s3r.compressed_attn_topk(q, kk, None, k, materialize_scores=False)
+    v = _randn((1, h, lk, 64), lk + 2, dtype).to(DEV)
+    _, idx_m, scores = s3r.compressed_attn_topk(q, kk, v, k, return_scores=True)
+    want = oracle.topk_from_scores(scores.cpu(), k)
+    np.testing.assert_array_equal(idx_m.cpu().numpy(), want)
+    np.testing.assert_array_equal(idx_f.cpu().numpy(), want)
+
+
 def test_fused_selection_special_scores():
     """Zero queries give all-zero scores (every column ties: indices 0..K-1); a huge key gives +inf scores."""
     lk = 200
