@@ -42,6 +42,10 @@ namespace bwd {
 using namespace sel;
 
 constexpr int kHalfBytes = 32 * 128;  // one half tile: 32 rows of 64 two-byte values
+// dK/dV at 16-token blocks: two neighbouring key blocks' lists are merged up to this many entries together (the union's
+// hash table has 512 slots, and with the merged list of 386 entries per wave four workgroups still fit a CU's LDS;
+// 128 / 256 / 384: 4.36 / 4.06 / 3.93 ms at 266 496 tokens, top-32, 4.40 without merging)
+constexpr int kMergeMax = 384;
 constexpr float kLog2e = 1.4426950408889634f;
 
 typedef std::integral_constant<int, 0> H0;
@@ -552,6 +556,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_g1[kTileBytes];
   __shared__ __attribute__((aligned(256))) float lds_s0[128];  // [0,64): lse of the tile's 64 queries, [64,128): delta
   __shared__ __attribute__((aligned(256))) float lds_s1[128];
+  __shared__ __attribute__((aligned(16))) int2 lds_union[BLK == 16 ? 2 : 1][BLK == 16 ? kMergeMax + 2 : 1];  // BLK 16: merged lists, per wave
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -593,10 +598,10 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
   const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
 
-  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks).  BLK 16: the wave takes its two
-  // key blocks one after the other, and lanes c and c + 16 both hold key c & 15 of the current block: each half of
-  // the lanes then meets its own 16-query block of the tile (two list entries per step), and the two halves' partial
-  // dK^T, dV^T are added up when the list ends.
+  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks).  BLK 16: 32 keys are two
+  // neighbouring key blocks A and B, whose lists name mostly the same query blocks: the wave walks the MERGED lists
+  // (both are ascending), two distinct query blocks per step, and every (query block, key block) quadrant of the
+  // 32 x 32 scores counts as often as that key block's list names the query block (0: not at all).
   int64_t key = (int64_t)kb * 64 + wave * 32 + c;
   V8 bk[4], bv[4];
   f32x16 dkt[2], dvt[2];  // dK^T, dV^T [dt]: lane = key, registers = head_dim
@@ -639,8 +644,12 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride;
     off16 = off;
   }
-  const int32_t* cur_list = list;  // BLK 16: list and length of the key block being processed
-  int cur_len = 0;
+  // BLK 16: the two lists being merged (key blocks A and B of the current 32 keys), read positions, and the weights of
+  // the step being computed
+  const int32_t* lst_a = list;
+  const int32_t* lst_b = list;
+  int len_a = 0, len_b = 0;
+  uint32_t step_w = 0;
   // BLK 16, two ways through the tile's four lists.  Workgroups of the first pass (long lists) share every list
   // between their two waves; in the second pass each wave walks the lists of its own two key blocks, without
   // barriers or hand-over, which is cheaper where the lists are short.
@@ -659,7 +668,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   auto block_of = [&](int i) -> int64_t {  // BLK 16: the list position itself
     if constexpr (DENSE) return (int64_t)i;
     else if constexpr (BLK == 64) return (int64_t)entry(list, n_lists, held_a, base_a, i);
-    else return (int64_t)(coop ? 2 * i + wave : i);  // shared list: the two waves take alternate steps
+    else return (int64_t)i;  // (BLK 16 walks its merged lists by itself, below)
   };
 
   const float scale = p.scale;
@@ -717,11 +726,9 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       staged_inf = wave == 0 && lane > last;  // query rows beyond Lq: lse = +inf, no probability
       staged_to = sb + 64 * wave + lane;
     } else {
-      // this wave's half of the tile: the 16 queries of entries 2t and 2t + 1 of the current list (past its end: any
-      // rows, lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
-      const int t = (int)qblk;
-      const int32_t ea = 2 * t < cur_len ? entry(cur_list, cur_len, held_a, base_a, 2 * t) : -1;
-      const int32_t eb = 2 * t + 1 < cur_len ? entry(cur_list, cur_len, held_a, base_a, 2 * t + 1) : -1;
+      // this wave's half of the tile: the 16 queries of each of the step's two query blocks (none: any rows,
+      // lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
+      const int32_t ea = (int32_t)(qblk & 0xffffffffLL), eb = (int32_t)(qblk >> 32);  // the step's two query blocks (-1: none)
       const int64_t sa = ea >= 0 ? (int64_t)ea * 16 : 0, sbk = eb >= 0 ? (int64_t)eb * 16 : 0;
       const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
       const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
@@ -782,10 +789,17 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       for (int r = 0; r < 16; r++)
         if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) s[r] = 0.f;
     }
-    if constexpr (BLK == 16) {  // registers 0..7 are queries of list A's block, 8..15 of list B's; this lane's key is in one
+    if constexpr (BLK == 16) {  // registers 0..7 are queries of the step's first query block, 8..15 of its second; this
+      // lane's key block lists each of them step_w byte (2 * entry + key block) times
+      const int g = c >> 4;
+      const uint32_t w0 = (step_w >> (8 * g)) & 0xffu, w1 = (step_w >> (16 + 8 * g)) & 0xffu;
 #pragma unroll
-      for (int r = 0; r < 16; r++)
-        if ((r >> 3) != (c >> 4)) s[r] = 0.f;
+      for (int r = 0; r < 16; r++) s[r] = (r < 8 ? w0 : w1) != 0 ? s[r] : 0.f;
+      if ((step_w & 0xfefefefeu) != 0) {  // (wave-uniform) a query block named more than once by one list
+        const float f0 = (float)w0, f1 = (float)w1;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] *= r < 8 ? f0 : f1;
+      }
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) {
@@ -882,7 +896,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   auto compute_tile = [&](int64_t qblk, auto bufc) {
     if constexpr (BLK == 64) {
       tile64(bufc);
-    } else {  // this wave's keys only meet the queries of its own half of the tile
+    } else {  // this wave's 32 keys against the 32 queries in its own half of the tile buffers
       f32x16 s0, dp0;
       V8 pb0[2], db0[2];
       stage_a(bufc, wave, s0, dp0);
@@ -926,32 +940,140 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
     store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
   } else {
-    // Both waves walk the list of each of the tile's four key blocks together: steps t = wave, wave + 2, ..., entries
-    // 2t and 2t + 1 per step, so a long list is shared by four 16-lane groups and the two waves stay in balance.  At
-    // the end of a list the second wave hands its partial sums over through LDS (the tile buffers are idle then).
-    for (int li = 0; li < (coop ? 4 : 2); li++) {
-      const int64_t kblk = (int64_t)kb * 4 + (coop ? li : 2 * wave + li);
+    // Two ways through a key block's list.
+    // Single: the wave holds ONE key block twice (lanes c and c + 16 carry key c & 15) and takes entries 2t and 2t + 1 of
+    // its list per step; the first copy of the keys counts for the first entry's queries, the second for the second's,
+    // and the two copies' partial sums are added when the list ends.  Half of every 32 x 32 product is unused.
+    // Merged: the wave holds TWO neighbouring key blocks A and B (32 different keys), whose lists name mostly the same
+    // query blocks (49 distinct ones for 2 x 32 entries at 266 496 tokens, top-32), and walks the union of the two
+    // lists, two distinct query blocks per step; every (query block, key block) quadrant counts as often as that key
+    // block's list names the query block.  The union comes from a 512-slot hash table in this wave's (idle) half of a
+    // tile buffer, built by all lanes: compare-and-swap on the query block, linear probing, 1 added to byte 0 (list A)
+    // or byte 1 (list B) of the slot's count; the occupied slots are compacted into lds_union, eight slots per lane,
+    // positions from ballots.  The steps then come in the table's order (fp32 summation order only).  Used where the
+    // two lists have at most kMergeMax entries together and are not shared with the other wave.
+    int2* const uni = lds_union[BLK == 16 ? wave : 0];
+    int n_union = -1, step_no = 0;  // n_union < 0: single
+    auto build_union = [&]() {
+      int32_t* const hkey = reinterpret_cast<int32_t*>(lds_q0 + wave * kHalfBytes);  // [512]
+      uint32_t* const hcnt = reinterpret_cast<uint32_t*>(lds_q0 + wave * kHalfBytes + 2048);  // [512]
+      reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
+      reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
+      reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
+      reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
+      const int total = len_a + len_b;
+      for (int i0 = 0; i0 < total; i0 += 64) {
+        const int i = i0 + lane;
+        bool active = i < total;
+        const int32_t e = active ? (i < len_a ? lst_a[i] : lst_b[i - len_a]) : 0;
+        const uint32_t one = i < len_a ? 1u : 256u;
+        uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
+        while (active) {
+          const int32_t old = atomicCAS(hkey + slot, -1, e);
+          if (old == -1 || old == e) {
+            atomicAdd(hcnt + slot, one);
+            active = false;
+          } else {
+            slot = (slot + 1) & 511u;
+          }
+        }
+      }
+      const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
+      const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
+      const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+      const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      uint32_t pos = 0;  // occupied slots of the lanes below
+      n_union = 0;
+#pragma unroll
+      for (int s8 = 0; s8 < 8; s8++) {
+        const uint64_t m = __ballot(ks8[s8] >= 0);
+        pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
+        n_union += __popcll(m);
+      }
+#pragma unroll
+      for (int s8 = 0; s8 < 8; s8++)
+        if (ks8[s8] >= 0) uni[pos++] = make_int2(ks8[s8], cs8[s8]);
+      if (lane == 0) uni[n_union] = make_int2(-1, 0);  // the partner of an odd last entry
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): table read, list written before the first transfer lands there
+    };
+    // The next step of this wave: two query blocks (packed for `fetch`; -1: none) and their four weights, byte
+    // 2 * entry + key block.  A shared list (coop, single): the two waves take alternate steps.
+    auto next_step = [&](int64_t& blocks, uint32_t& w) -> bool {
+      const int t = step_no++;
+      int32_t q0, q1;
+      if (n_union >= 0) {  // merged: entries 2t, 2t + 1 of the union
+        if (2 * t >= n_union) return false;
+        const int4 v = *reinterpret_cast<const int4*>(uni + 2 * t);
+        q0 = __builtin_amdgcn_readfirstlane(v.x);
+        q1 = __builtin_amdgcn_readfirstlane(v.z);
+        const uint32_t c0 = (uint32_t)__builtin_amdgcn_readfirstlane(v.y), c1 = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
+        w = (c0 & 0xffffu) | (c1 << 16);
+      } else {  // single: entries 2u, 2u + 1 of the list; first key copy x first entry, second copy x second entry
+        const int u = coop ? 2 * t + wave : t;
+        if (2 * u >= len_a) return false;
+        q0 = entry(lst_a, len_a, held_a, base_a, 2 * u);
+        q1 = 2 * u + 1 < len_a ? entry(lst_a, len_a, held_a, base_a, 2 * u + 1) : -1;
+        w = 0x01000001u;
+      }
+      blocks = (int64_t)(uint32_t)q0 | ((int64_t)q1 << 32);
+      return true;
+    };
+    auto walk16 = [&]() {  // all steps of the current unit, double buffered
+      int64_t cur = 0, nxt = 0;
+      uint32_t wcur = 0, wnxt = 0;
+      if (!next_step(cur, wcur)) return;
+      fetch(cur, H0{});
+      while (true) {
+        sync();
+        const bool more1 = next_step(nxt, wnxt);
+        if (more1) fetch(nxt, H1{});
+        step_w = wcur;
+        compute_tile(cur, H0{});
+        if (!more1) break;
+        sync();
+        const bool more2 = next_step(cur, wcur);
+        if (more2) fetch(cur, H0{});
+        step_w = wnxt;
+        compute_tile(nxt, H1{});
+        if (!more2) break;
+      }
+    };
+    // Workgroups of the long-list pass: both waves walk the list of each of the tile's four key blocks together
+    // (single, alternate steps), so a long list is shared and the two waves stay in balance; at the end of a list the
+    // second wave hands its partial sums over through LDS (the tile buffers are idle then).  Otherwise each wave takes
+    // its own two key blocks: merged where their lists are short enough, else one after the other.
+    const int64_t nkb16 = (Lk + 15) >> 4;
+    const int64_t first = (int64_t)kb * 4 + (coop ? 0 : 2 * wave);
+    bool merged = false;
+    if (!coop && first + 1 < nkb16) merged = __builtin_amdgcn_readfirstlane(off16[first + 2] - off16[first]) <= kMergeMax;
+    const int n_units = coop ? 4 : (merged ? 1 : 2);
+    for (int li = 0; li < n_units; li++) {
+      const int64_t kblk = first + li;  // key block A; merged: B = A + 1
       if (kblk * 16 >= Lk) break;  // no such key block (shared lists: the same for both waves)
-      key = kblk * 16 + (c & 15);
-      const int32_t lo = __builtin_amdgcn_readfirstlane(off16[kblk]), hi = __builtin_amdgcn_readfirstlane(off16[kblk + 1]);
-      cur_list = list + lo;
-      cur_len = hi - lo;
-      const int steps = (cur_len + 1) >> 1;               // of the list
-      n_lists = coop ? (steps - wave + 1) >> 1 : steps;   // of this wave
+      key = merged ? kblk * 16 + c : kblk * 16 + (c & 15);
+      const int32_t oa = __builtin_amdgcn_readfirstlane(off16[kblk]), ob = __builtin_amdgcn_readfirstlane(off16[kblk + 1]);
+      lst_a = list + oa;
+      len_a = ob - oa;
+      lst_b = list + ob;
+      len_b = merged ? __builtin_amdgcn_readfirstlane(off16[kblk + 2]) - ob : 0;
       held_a = -1;
       base_a = -64;
+      step_no = 0;
+      n_union = -1;
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's last LDS reads are done before new transfers land
+      if (merged) build_union();
       load_keys();
-      walk();
-      // lanes c and c + 16 hold partial sums for the same key
+      walk16();
+      if (!merged) {  // lanes c and c + 16 hold partial sums for the same key
 #pragma unroll
-      for (int dt = 0; dt < 2; dt++)
+        for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          dkt[dt][r] += __shfl_xor(dkt[dt][r], 16);
-          dvt[dt][r] += __shfl_xor(dvt[dt][r], 16);
-        }
-      const bool live = c < 16 && key < Lk;
+          for (int r = 0; r < 16; r++) {
+            dkt[dt][r] += __shfl_xor(dkt[dt][r], 16);
+            dvt[dt][r] += __shfl_xor(dvt[dt][r], 16);
+          }
+      }
+      const bool live = (merged || c < 16) && key < Lk;
       if (!coop) {
         store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
         store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
