@@ -42,9 +42,8 @@ namespace bwd {
 using namespace sel;
 
 constexpr int kHalfBytes = 32 * 128;  // one half tile: 32 rows of 64 two-byte values
-// dK/dV at 16-token blocks: two neighbouring key blocks' lists are merged up to this many entries together (the union's
-// hash table has 512 slots, and with the merged list of 386 entries per wave four workgroups still fit a CU's LDS;
-// 128 / 256 / 384: 4.36 / 4.06 / 3.93 ms at 266 496 tokens, top-32, 4.40 without merging)
+// dK/dV at 16-token blocks: entries per chunk of the union of two neighbouring key blocks' lists (half from each list;
+// the union's hash table has 512 slots, and with a list of 386 entries per wave four workgroups still fit a CU's LDS)
 constexpr int kMergeMax = 384;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -940,85 +939,103 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
     store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
   } else {
-    // Two ways through a key block's list.
-    // Single: the wave holds ONE key block twice (lanes c and c + 16 carry key c & 15) and takes entries 2t and 2t + 1 of
-    // its list per step; the first copy of the keys counts for the first entry's queries, the second for the second's,
-    // and the two copies' partial sums are added when the list ends.  Half of every 32 x 32 product is unused.
-    // Merged: the wave holds TWO neighbouring key blocks A and B (32 different keys), whose lists name mostly the same
-    // query blocks (49 distinct ones for 2 x 32 entries at 266 496 tokens, top-32), and walks the union of the two
-    // lists, two distinct query blocks per step; every (query block, key block) quadrant counts as often as that key
-    // block's list names the query block.  The union comes from a 512-slot hash table in this wave's (idle) half of a
-    // tile buffer, built by all lanes: compare-and-swap on the query block, linear probing, 1 added to byte 0 (list A)
-    // or byte 1 (list B) of the slot's count; the occupied slots are compacted into lds_union, eight slots per lane,
-    // positions from ballots.  The steps then come in the table's order (fp32 summation order only).  Used where the
-    // two lists have at most kMergeMax entries together and are not shared with the other wave.
-    int2* const uni = lds_union[BLK == 16 ? wave : 0];
-    int n_union = -1, step_no = 0;  // n_union < 0: single
-    auto build_union = [&]() {
-      int32_t* const hkey = reinterpret_cast<int32_t*>(lds_q0 + wave * kHalfBytes);  // [512]
-      uint32_t* const hcnt = reinterpret_cast<uint32_t*>(lds_q0 + wave * kHalfBytes + 2048);  // [512]
-      reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
-      reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
-      reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
-      reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
-      const int total = len_a + len_b;
-      for (int i0 = 0; i0 < total; i0 += 64) {
-        const int i = i0 + lane;
-        bool active = i < total;
-        const int32_t e = active ? (i < len_a ? lst_a[i] : lst_b[i - len_a]) : 0;
-        const uint32_t one = i < len_a ? 1u : 256u;
-        uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
-        while (active) {
-          const int32_t old = atomicCAS(hkey + slot, -1, e);
-          if (old == -1 || old == e) {
-            atomicAdd(hcnt + slot, one);
-            active = false;
-          } else {
-            slot = (slot + 1) & 511u;
+    // The wave holds TWO neighbouring key blocks A and B (32 different keys), whose lists name mostly the same query
+    // blocks (49 distinct ones for 2 x 32 entries at 266 496 tokens, top-32), and walks the UNION of the two lists, two
+    // distinct query blocks per step; every (query block, key block) quadrant of the 32 x 32 scores counts as often as
+    // that key block's list names the query block (0: not at all).  The union is built a chunk at a time: up to kChunk
+    // entries of list A, and the entries of list B below the first value A has left (both lists are ascending, so
+    // these are the entries that can meet this chunk of A), up to kChunk as well.  A chunk's entries go into a 512-slot
+    // hash table in an idle half of a tile buffer, by all lanes: compare-and-swap on the query block, linear probing, 1
+    // added to byte 0 (list A) or byte 1 (list B) of the slot's count; the occupied slots are compacted into lds_union,
+    // eight slots per lane, positions from ballots.  The steps come in the table's order (fp32 summation order only).
+    // Every list entry is in exactly one chunk, so whatever the chunks' borders, every (query block, key block) pair
+    // is counted as often as listed.  A pair of lists shared by the two waves (coop): wave 0 builds, both walk.
+    constexpr int kChunk = kMergeMax / 2;
+    int2* const uni = lds_union[BLK == 16 && !coop ? wave : 0];
+    int n_union = 0, step_no = 0, pa = 0, pb = 0;
+    auto build_chunk = [&]() -> bool {
+      const int na = len_a - pa < kChunk ? len_a - pa : kChunk;
+      const int32_t tau = pa + na < len_a ? __builtin_amdgcn_readfirstlane(lst_a[pa + na]) : 0x7fffffff;
+      int32_t bval[kChunk / 64];
+      int nb = 0;
+#pragma unroll
+      for (int jw = 0; jw < kChunk / 64; jw++) {
+        const int i = pb + 64 * jw + lane;
+        bval[jw] = i < len_b ? lst_b[i] : 0x7fffffff;
+        nb += __popcll(__ballot(bval[jw] < tau));  // a prefix of the window: the list is ascending
+      }
+      if (na + nb == 0) return false;
+      if (!coop || wave == 0) {
+        int32_t* const hkey = reinterpret_cast<int32_t*>(lds_q0 + wave * kHalfBytes);  // [512]
+        uint32_t* const hcnt = reinterpret_cast<uint32_t*>(lds_q0 + wave * kHalfBytes + 2048);  // [512]
+        reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
+        reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
+        reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
+        reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
+        auto insert = [&](bool active, int32_t e, uint32_t one) {
+          uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
+          while (active) {
+            const int32_t old = atomicCAS(hkey + slot, -1, e);
+            if (old == -1 || old == e) {
+              atomicAdd(hcnt + slot, one);
+              active = false;
+            } else {
+              slot = (slot + 1) & 511u;
+            }
           }
+        };
+#pragma unroll
+        for (int jw = 0; jw < kChunk / 64; jw++) {
+          const int i = 64 * jw + lane;
+          const bool act = i < na;
+          insert(act, act ? lst_a[pa + i] : 0, 1u);
         }
-      }
-      const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
-      const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
-      const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-      const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-      uint32_t pos = 0;  // occupied slots of the lanes below
-      n_union = 0;
 #pragma unroll
-      for (int s8 = 0; s8 < 8; s8++) {
-        const uint64_t m = __ballot(ks8[s8] >= 0);
-        pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
-        n_union += __popcll(m);
-      }
+        for (int jw = 0; jw < kChunk / 64; jw++) insert(64 * jw + lane < nb, bval[jw], 256u);
+        const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
+        const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
+        const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        uint32_t pos = 0;  // occupied slots of the lanes below
+        n_union = 0;
 #pragma unroll
-      for (int s8 = 0; s8 < 8; s8++)
-        if (ks8[s8] >= 0) uni[pos++] = make_int2(ks8[s8], cs8[s8]);
-      if (lane == 0) uni[n_union] = make_int2(-1, 0);  // the partner of an odd last entry
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): table read, list written before the first transfer lands there
+        for (int s8 = 0; s8 < 8; s8++) {
+          const uint64_t m = __ballot(ks8[s8] >= 0);
+          pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
+          n_union += __popcll(m);
+        }
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++)
+          if (ks8[s8] >= 0) uni[pos++] = make_int2(ks8[s8], cs8[s8]);
+        if (lane == 0) {
+          uni[n_union] = make_int2(-1, 0);      // the partner of an odd last entry
+          uni[kMergeMax + 1] = make_int2(n_union, 0);  // for the other wave of a shared pair
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): table read, list written before the first transfer lands there
+      }
+      pa += na;
+      pb += nb;
+      if (coop) {
+        __syncthreads();
+        n_union = __builtin_amdgcn_readfirstlane(uni[kMergeMax + 1].x);
+      }
+      step_no = 0;
+      return true;
     };
-    // The next step of this wave: two query blocks (packed for `fetch`; -1: none) and their four weights, byte
-    // 2 * entry + key block.  A shared list (coop, single): the two waves take alternate steps.
+    // The next step of this wave: entries 2t, 2t + 1 of the chunk's union as two query blocks (packed for `fetch`; -1:
+    // none) and their four weights, byte 2 * entry + key block.  A shared pair: the two waves take alternate steps.
     auto next_step = [&](int64_t& blocks, uint32_t& w) -> bool {
-      const int t = step_no++;
-      int32_t q0, q1;
-      if (n_union >= 0) {  // merged: entries 2t, 2t + 1 of the union
-        if (2 * t >= n_union) return false;
-        const int4 v = *reinterpret_cast<const int4*>(uni + 2 * t);
-        q0 = __builtin_amdgcn_readfirstlane(v.x);
-        q1 = __builtin_amdgcn_readfirstlane(v.z);
-        const uint32_t c0 = (uint32_t)__builtin_amdgcn_readfirstlane(v.y), c1 = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
-        w = (c0 & 0xffffu) | (c1 << 16);
-      } else {  // single: entries 2u, 2u + 1 of the list; first key copy x first entry, second copy x second entry
-        const int u = coop ? 2 * t + wave : t;
-        if (2 * u >= len_a) return false;
-        q0 = entry(lst_a, len_a, held_a, base_a, 2 * u);
-        q1 = 2 * u + 1 < len_a ? entry(lst_a, len_a, held_a, base_a, 2 * u + 1) : -1;
-        w = 0x01000001u;
-      }
+      const int t = coop ? 2 * step_no + wave : step_no;
+      step_no++;
+      if (2 * t >= n_union) return false;
+      const int4 v = *reinterpret_cast<const int4*>(uni + 2 * t);
+      const int32_t q0 = __builtin_amdgcn_readfirstlane(v.x), q1 = __builtin_amdgcn_readfirstlane(v.z);
+      const uint32_t c0 = (uint32_t)__builtin_amdgcn_readfirstlane(v.y), c1 = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
+      w = (c0 & 0xffffu) | (c1 << 16);
       blocks = (int64_t)(uint32_t)q0 | ((int64_t)q1 << 32);
       return true;
     };
-    auto walk16 = [&]() {  // all steps of the current unit, double buffered
+    auto walk16 = [&]() {  // all steps of the current chunk, double buffered
       int64_t cur = 0, nxt = 0;
       uint32_t wcur = 0, wnxt = 0;
       if (!next_step(cur, wcur)) return;
@@ -1038,42 +1055,30 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         if (!more2) break;
       }
     };
-    // Workgroups of the long-list pass: both waves walk the list of each of the tile's four key blocks together
-    // (single, alternate steps), so a long list is shared and the two waves stay in balance; at the end of a list the
-    // second wave hands its partial sums over through LDS (the tile buffers are idle then).  Otherwise each wave takes
-    // its own two key blocks: merged where their lists are short enough, else one after the other.
+    // Workgroups of the long-list pass: both waves walk each of the tile's two pairs of key blocks together (alternate
+    // steps), so a long list is shared and the two waves stay in balance; at the end of a pair the second wave hands its
+    // partial sums over through LDS (the tile buffers are idle then).  Otherwise each wave takes its own pair.
     const int64_t nkb16 = (Lk + 15) >> 4;
-    const int64_t first = (int64_t)kb * 4 + (coop ? 0 : 2 * wave);
-    bool merged = false;
-    if (!coop && first + 1 < nkb16) merged = __builtin_amdgcn_readfirstlane(off16[first + 2] - off16[first]) <= kMergeMax;
-    const int n_units = coop ? 4 : (merged ? 1 : 2);
-    for (int li = 0; li < n_units; li++) {
-      const int64_t kblk = first + li;  // key block A; merged: B = A + 1
-      if (kblk * 16 >= Lk) break;  // no such key block (shared lists: the same for both waves)
-      key = merged ? kblk * 16 + c : kblk * 16 + (c & 15);
+    for (int li = 0; li < (coop ? 2 : 1); li++) {
+      const int64_t kblk = (int64_t)kb * 4 + 2 * (coop ? li : wave);  // key block A; B = A + 1 (may not exist)
+      if (kblk * 16 >= Lk) break;  // no such key blocks (shared pairs: the same for both waves)
+      key = kblk * 16 + c;
       const int32_t oa = __builtin_amdgcn_readfirstlane(off16[kblk]), ob = __builtin_amdgcn_readfirstlane(off16[kblk + 1]);
       lst_a = list + oa;
       len_a = ob - oa;
       lst_b = list + ob;
-      len_b = merged ? __builtin_amdgcn_readfirstlane(off16[kblk + 2]) - ob : 0;
-      held_a = -1;
-      base_a = -64;
-      step_no = 0;
-      n_union = -1;
+      len_b = kblk + 1 < nkb16 ? __builtin_amdgcn_readfirstlane(off16[kblk + 2]) - ob : 0;
+      pa = pb = 0;
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's last LDS reads are done before new transfers land
-      if (merged) build_union();
       load_keys();
-      walk16();
-      if (!merged) {  // lanes c and c + 16 hold partial sums for the same key
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            dkt[dt][r] += __shfl_xor(dkt[dt][r], 16);
-            dvt[dt][r] += __shfl_xor(dvt[dt][r], 16);
-          }
+      while (build_chunk()) {
+        walk16();
+        if (coop) {
+          __builtin_amdgcn_s_waitcnt(0xC07F);
+          __syncthreads();  // both waves are through the chunk before its list and the table's buffer are reused
+        }
       }
-      const bool live = (merged || c < 16) && key < Lk;
+      const bool live = key < Lk;
       if (!coop) {
         store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
         store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
