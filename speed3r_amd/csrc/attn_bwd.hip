@@ -27,13 +27,14 @@
 // never read (transfers re-read the last valid row).
 //
 // 16-token blocks (BLK = 16, the reference layer's own block size) run through the same kernels: a 32-row half tile
-// is then two 16-row blocks.  dQ kernel: query blocks 2h, 2h+1 of the wave's 64 queries and entry t of each one's
-// index list; key half h only meets query half h, so the other half's products are not issued.  dK/dV kernel: a wave
-// takes one 16-key block at a time, held twice (lanes c and c + 16 carry key c & 15), against entries 2t and 2t + 1 of
-// that block's query-block list, and adds the two halves' partial sums when the list ends.  Either way the wanted
-// 16 x 16 blocks sit on the diagonal of a 32 x 32 product and the other two quadrants get P = 0.  Tiles whose lists
-// are long (first pass of the grid) share every list between the workgroup's two waves, which hand partial sums over
-// through LDS; the other tiles give each wave two key blocks of its own.
+// is then two 16-row blocks, and neighbouring blocks name mostly the same partners, so both kernels walk UNIONS of
+// lists (distinct blocks from a 512-slot hash table in LDS, with a count byte per list: how often that list names the
+// block; a product's quadrant whose count is 0 gets P = 0, one listed twice counts twice).  dQ kernel: the union of
+// the index rows of the wave's four query blocks, two distinct key blocks per half tile against all 64 queries.
+// dK/dV kernel: a wave holds two neighbouring 16-key blocks (one key per lane again) and walks the union of their two
+// query-block lists, two entries per step, built a chunk of the (ascending) lists at a time.  Tiles whose lists are
+// long (first pass of the grid) share every pair of lists between the workgroup's two waves, which take alternate
+// steps and hand partial sums over through LDS; the other tiles give each wave a pair of key blocks of its own.
 #include "select_common.h"
 #include "attn_bwd.h"
 
