@@ -31,10 +31,9 @@
 // lists (distinct blocks from a 512-slot hash table in LDS, with a count byte per list: how often that list names the
 // block; a product's quadrant whose count is 0 gets P = 0, one listed twice counts twice).  dQ kernel: the union of
 // the index rows of the wave's four query blocks, two distinct key blocks per half tile against all 64 queries.
-// dK/dV kernel: a wave holds two neighbouring 16-key blocks (one key per lane again) and walks the union of their two
-// query-block lists, two entries per step, built a chunk of the (ascending) lists at a time.  Tiles whose lists are
-// long (first pass of the grid) share every pair of lists between the workgroup's two waves, which take alternate
-// steps and hand partial sums over through LDS; the other tiles give each wave a pair of key blocks of its own.
+// dK/dV kernel: the workgroup's 64 keys are four neighbouring key blocks; it walks the union of their four
+// query-block lists, four entries per 64-row tile, with the tile code of the 64-token blocks; the union is built a
+// chunk of the (ascending) lists at a time.
 #include "select_common.h"
 #include "attn_bwd.h"
 
@@ -43,8 +42,8 @@ namespace bwd {
 using namespace sel;
 
 constexpr int kHalfBytes = 32 * 128;  // one half tile: 32 rows of 64 two-byte values
-// dK/dV at 16-token blocks: entries per chunk of the union of two neighbouring key blocks' lists (half from each list;
-// the union's hash table has 512 slots, and with a list of 386 entries per wave four workgroups still fit a CU's LDS)
+// dK/dV at 16-token blocks: list entries per chunk of the union of four neighbouring key blocks' lists (a quarter from
+// each list; the union's hash table has 512 slots)
 constexpr int kMergeMax = 384;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -554,9 +553,14 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_q1[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_g0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char lds_g1[kTileBytes];
-  __shared__ __attribute__((aligned(256))) float lds_s0[128];  // [0,64): lse of the tile's 64 queries, [64,128): delta
-  __shared__ __attribute__((aligned(256))) float lds_s1[128];
-  __shared__ __attribute__((aligned(16))) int2 lds_union[BLK == 16 ? 2 : 1][BLK == 16 ? kMergeMax + 2 : 1];  // BLK 16: merged lists, per wave
+  // per-query scalars of a tile: [0,64) lse, [64,128) delta.  BLK 16: four such pairs kVar floats apart, one per key
+  // block of the workgroup, each with its own variant of lse (delta is repeated, so that a lane finds both values of
+  // a query at a fixed distance and reads them with one instruction)
+  constexpr int kVar = 136;
+  constexpr int kDeltaAt = 64;
+  __shared__ __attribute__((aligned(256))) float lds_s0[BLK == 16 ? 4 * kVar : 128];
+  __shared__ __attribute__((aligned(256))) float lds_s1[BLK == 16 ? 4 * kVar : 128];
+  __shared__ __attribute__((aligned(16))) int2 lds_union[BLK == 16 ? kMergeMax + 8 : 1];  // BLK 16: the current chunk's union of the four lists
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -598,11 +602,9 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   const float* lsep = p.lse + ((int64_t)b * p.H + h) * Lq;
   const float* dlp = p.delta + ((int64_t)b * p.H + h) * Lq;
 
-  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks).  BLK 16: 32 keys are two
-  // neighbouring key blocks A and B, whose lists name mostly the same query blocks: the wave walks the MERGED lists
-  // (both are ascending), two distinct query blocks per step, and every (query block, key block) quadrant of the
-  // 32 x 32 scores counts as often as that key block's list names the query block (0: not at all).
-  int64_t key = (int64_t)kb * 64 + wave * 32 + c;
+  // B operands K and V of this wave's 32 keys (lane = key, head_dim chunk hh + 2 ks).  BLK 16: these are two
+  // neighbouring key blocks, the workgroup's 64 keys four.
+  const int64_t key = (int64_t)kb * 64 + wave * 32 + c;
   V8 bk[4], bv[4];
   f32x16 dkt[2], dvt[2];  // dK^T, dV^T [dt]: lane = key, registers = head_dim
   auto load_keys = [&]() {
@@ -623,7 +625,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 #pragma unroll
       for (int r = 0; r < 16; r++) { dkt[dt][r] = 0.f; dvt[dt][r] = 0.f; }
   };
-  if constexpr (BLK == 64) load_keys();
+  load_keys();
 
   // query blocks that attend to this key block
   static_assert(BLK == 64 || (BLK == 16 && !DENSE), "blocks of 64 tokens, or of 16 with key-centric lists");
@@ -644,16 +646,9 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     list = p.kq_list + ((int64_t)b * p.H + h) * p.list_stride;
     off16 = off;
   }
-  // BLK 16: the two lists being merged (key blocks A and B of the current 32 keys), read positions, and the weights of
-  // the step being computed
-  const int32_t* lst_a = list;
-  const int32_t* lst_b = list;
-  int len_a = 0, len_b = 0;
-  uint32_t step_w = 0;
-  // BLK 16, two ways through the tile's four lists.  Workgroups of the first pass (long lists) share every list
-  // between their two waves; in the second pass each wave walks the lists of its own two key blocks, without
-  // barriers or hand-over, which is cheaper where the lists are short.
-  const bool coop = BLK == 16 && long_pass;
+  // BLK 16: how often each of the workgroup's four key blocks lists the two query blocks this wave fetches for the
+  // tile in flight (a byte per key block), set by block_of for the fetch that follows it
+  uint32_t ent_cnt_a = 0, ent_cnt_b = 0;
   // List entries come 64 at a time (lane l holds entry base + l), so the latency of the list read is paid once per
   // 64 tiles and not in front of every tile's transfers.  The lists are walked front to back.
   int32_t held_a = -1;
@@ -665,33 +660,42 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     }
     return __builtin_amdgcn_readlane(held, i - base);
   };
-  auto block_of = [&](int i) -> int64_t {  // BLK 16: the list position itself
-    if constexpr (DENSE) return (int64_t)i;
-    else if constexpr (BLK == 64) return (int64_t)entry(list, n_lists, held_a, base_a, i);
-    else return (int64_t)i;  // (BLK 16 walks its merged lists by itself, below)
+  auto block_of = [&](int i) -> int64_t {
+    if constexpr (DENSE) {
+      return (int64_t)i;
+    } else if constexpr (BLK == 64) {
+      return (int64_t)entry(list, n_lists, held_a, base_a, i);
+    } else {  // tile i of the chunk: entries 4i .. 4i+3 of the union, this wave fetches 4i + 2 wave and the next one
+      const int4 v = *reinterpret_cast<const int4*>(lds_union + 4 * i + 2 * wave);
+      const int32_t q0 = __builtin_amdgcn_readfirstlane(v.x), q1 = __builtin_amdgcn_readfirstlane(v.z);
+      ent_cnt_a = (uint32_t)__builtin_amdgcn_readfirstlane(v.y);
+      ent_cnt_b = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
+      return (int64_t)(uint32_t)q0 | ((int64_t)q1 << 32);  // packed for `fetch`; -1: none
+    }
   };
 
   const float scale = p.scale;
   const float sl2 = scale * kLog2e;
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
+  const int lse_at = BLK == 16 ? (2 * wave + (c >> 4)) * kVar : 0;
   // (one per parity of the instruction inside its half tile: the chunk map of rows 8..15 differs from that of rows 0..7)
   const uint32_t q_voff[2] = {(uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16),
                               (uint32_t)(lane >> 3) * qrow + (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
   const uint32_t g_voff[2] = {(uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ k_swizzle(lane >> 3)) * 16),
                               (uint32_t)(lane >> 3) * grow + (uint32_t)(((lane & 7) ^ k_swizzle((lane >> 3) + 8)) * 16)};
 
-  float staged = 0.f;          // this lane's lse (wave 0) or delta (wave 1) value of the tile in flight, as loaded
-  float staged_by = 1.f;       // the factor it is published with
-  bool staged_inf = false;     // BLK 16: rows past the end of a block publish lse = +inf
-  float* staged_to = nullptr;  // where it goes in LDS
+  float staged = 0.f;          // this lane's lse or delta value of the tile in flight, as loaded (BLK 64: wave 0 lse,
+                               // wave 1 delta; BLK 16: lanes 0..31 lse, 32..63 delta of the wave's 32 queries)
+  bool staged_inf = false;     // rows past the end of the tensor or of a block publish lse = +inf
+  uint32_t staged_cnt = 0;     // BLK 16: the count bytes of the row's query block
+  int staged_buf = -1;         // (wave-uniform) the buffer it goes to; -1: nothing staged
   // One query tile (64 rows of Q and dO, 64 lse and delta values) -> buffer BUF; each wave moves half of every
   // operand (instructions 2*wave, 2*wave+1 of both 32-row halves), wave 0 the lse values, wave 1 delta.
   auto fetch = [&](int64_t qblk, auto bufc) {
     constexpr int BUF = decltype(bufc)::value;
     char* qb = reinterpret_cast<char*>(BUF == 0 ? lds_q0 : lds_q1);
     char* gb = reinterpret_cast<char*>(BUF == 0 ? lds_g0 : lds_g1);
-    float* sb = BUF == 0 ? lds_s0 : lds_s1;
     if constexpr (BLK == 64) {
       const int64_t start = qblk * 64;
       const int last = (int)((Lq - start < 64 ? Lq - start : 64) - 1);
@@ -718,13 +722,12 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
           dma_rows<E, true>(gp + start * p.sgm, grow, 32 * hf, last, gb + hf * kHalfBytes, lane, 2 * wave, 2 * wave + 2);
         }
       }
-      // per-query scalars pass through a register: they are scaled once here (lse to base 2, delta by the softmax
-      // scale) instead of once per score, and stored to LDS by `publish` before the barrier that opens the tile
+      // per-query scalars pass through a register and are stored to LDS by `publish` before the barrier that opens
+      // the tile
       const int r = lane < last ? lane : last;
       staged = ((wave == 0 ? lsep : dlp) + start)[r];
-      staged_by = wave == 0 ? kLog2e : scale;
       staged_inf = wave == 0 && lane > last;  // query rows beyond Lq: lse = +inf, no probability
-      staged_to = sb + 64 * wave + lane;
+      staged_buf = BUF;
     } else {
       // this wave's half of the tile: the 16 queries of each of the step's two query blocks (none: any rows,
       // lse = +inf); lanes 0..31 fetch the 32 lse values, lanes 32..63 the delta values
@@ -733,96 +736,69 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
       const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
       const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
-      dma_rows16<E, true>(qp + sa * p.sqm, qp + sbk * p.sqm, qrow, la, lb, qb + wave * kHalfBytes, lane);
-      dma_rows16<E, true>(gp + sa * p.sgm, gp + sbk * p.sgm, grow, la, lb, gb + wave * kHalfBytes, lane);
+      if (na == 16 && nb == 16) {
+        // (wave-uniform) two full blocks: the per-lane offsets of a full tile serve (the chunk map ignores row bit 4),
+        // rows 8..15 of a block ride in the scalar offset
+        const __amdgpu_buffer_rsrc_t rqa = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + sa * p.sqm), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rqb = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + sbk * p.sqm), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rga = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + sa * p.sgm), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rgb = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + sbk * p.sgm), 0, 0x7fffffff, 0x00020000);
+        char* qh = qb + wave * kHalfBytes;
+        char* gh = gb + wave * kHalfBytes;
+        // the per-lane offsets are made here, from a copy of the lane number the compiler cannot see through: kept
+        // across the tile's work they would cost the four registers that the tile code has not got
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const uint32_t ch[2] = {(uint32_t)(((ln & 7) ^ k_swizzle(ln >> 3)) * 16), (uint32_t)(((ln & 7) ^ k_swizzle((ln >> 3) + 8)) * 16)};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? rqa : rqb, (__attribute__((address_space(3))) void*)(qh + i * 1024), 16,
+                                                   (uint32_t)(ln >> 3) * qrow + ch[i & 1], (i & 1) * 8 * qrow, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? rga : rgb, (__attribute__((address_space(3))) void*)(gh + i * 1024), 16,
+                                                   (uint32_t)(ln >> 3) * grow + ch[i & 1], (i & 1) * 8 * grow, 0, 0);
+        }
+      } else {
+        dma_rows16<E, true>(qp + sa * p.sqm, qp + sbk * p.sqm, qrow, la, lb, qb + wave * kHalfBytes, lane);
+        dma_rows16<E, true>(gp + sa * p.sgm, gp + sbk * p.sgm, grow, la, lb, gb + wave * kHalfBytes, lane);
+      }
       const int j = lane & 31, j16 = j & 15;
       const bool second = (j >> 4) != 0;
       const int nmine = second ? nb : na;
       const int64_t row = (second ? sbk : sa) + (j16 < nmine ? j16 : 0);
       staged = (hh == 0 ? lsep : dlp)[row];
-      staged_by = hh == 0 ? kLog2e : scale;
       staged_inf = hh == 0 && j16 >= nmine;
-      staged_to = sb + 64 * hh + 32 * wave + j;
+      staged_cnt = second ? ent_cnt_b : ent_cnt_a;
+      staged_buf = BUF;
     }
   };
   // The loaded value is first touched here, a whole tile of work after its load: any arithmetic on it inside `fetch`
   // would make the wave wait for the load there, and with it (the counter is in order) for the tile transfers issued
   // just before, which is the tile that should be in flight during the current tile's work.
   auto publish = [&]() {
-    if (staged_to != nullptr) *staged_to = staged_inf ? INFINITY : staged * staged_by;
-    staged_to = nullptr;
-  };
-  // One tile in three stages per 32-query half, issued so that the matrix products of one half run under the
-  // vector work of the other: A = row reads + S, dP; B = P and dS from the per-query scalars; C = transposed reads +
-  // dV^T, dK^T.
-  auto stage_a = [&](auto bufc, const int HF, f32x16& s, f32x16& dp) {
-    constexpr int BUF = decltype(bufc)::value;
-    const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
-    const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
-    V8 aq[4], ag[4];
-    read_rows<E, true>(qb, c, hh, aq);
-    read_rows<E, true>(gb, c, hh, ag);
+    if (staged_buf < 0) return;
+    float* const sb = staged_buf == 0 ? lds_s0 : lds_s1;
+    if constexpr (BLK == 64) {
+      // scaled once here (lse to base 2, delta by the softmax scale) instead of once per score
+      sb[64 * wave + lane] = staged_inf ? INFINITY : staged * (wave == 0 ? kLog2e : scale);
+    } else {
+      // P of (query, key) counts as often as the key's block lists the query's block: the count goes into the
+      // exponent (lse - log2(count); 0 times: lse = +inf), one variant of the query's value per key block
+      const bool is_lse = hh == 0;
+      const float base = staged_inf ? INFINITY : staged * (is_lse ? kLog2e : scale);
+      const bool plain = __ballot(is_lse && (staged_cnt & 0xfefefefeu) != 0) == 0;  // (wave-uniform) no block listed twice
+      float* const to = sb + (is_lse ? 0 : kDeltaAt) + 32 * wave + (lane & 31);
 #pragma unroll
-    for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) s = Mma<E>::mma(aq[ks], bk[ks], s);    // S[q][key]: registers = queries, lane = key
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(ag[ks], bv[ks], dp);  // dP[q][key]
-  };
-  auto stage_b = [&](int64_t qblk, auto bufc, const int HF, f32x16& s, f32x16& dp, V8 (&pb)[2], V8 (&db)[2]) {
-    constexpr int BUF = decltype(bufc)::value;
-    const float* sb = (BUF == 0 ? lds_s0 : lds_s1) + 32 * HF;
-    const int nvalid = BLK == 64 ? (int)(Lq - qblk * 64 < 64 ? Lq - qblk * 64 : 64) : 64;  // BLK 16: lse = +inf does it
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sb + 4 * hh + 8 * j);        // queries 4hh + 8j + {0..3} of the half
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sb + 64 + 4 * hh + 8 * j);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int r = 4 * j + i;
-        s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], sl2, -l4[i]));  // P (l4: lse in base 2)
-        dp[r] = fmaf(dp[r], scale, -d4[i]);                     // scale * (dP - delta) (d4: delta * scale)
+      for (int kk = 0; kk < 4; kk++) {
+        const uint32_t wgt = (staged_cnt >> (8 * kk)) & 0xffu;
+        float vkk = is_lse && wgt == 0 ? INFINITY : base;
+        if (!plain && is_lse) vkk -= __builtin_amdgcn_logf((float)(wgt > 1 ? wgt : 1));
+        to[kk * kVar] = vkk;
       }
     }
-    if (nvalid < 64) {  // query rows beyond Lq carry no probability
-#pragma unroll
-      for (int r = 0; r < 16; r++)
-        if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) s[r] = 0.f;
-    }
-    if constexpr (BLK == 16) {  // registers 0..7 are queries of the step's first query block, 8..15 of its second; this
-      // lane's key block lists each of them step_w byte (2 * entry + key block) times
-      const int g = c >> 4;
-      const uint32_t w0 = (step_w >> (8 * g)) & 0xffu, w1 = (step_w >> (16 + 8 * g)) & 0xffu;
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[r] = (r < 8 ? w0 : w1) != 0 ? s[r] : 0.f;
-      if ((step_w & 0xfefefefeu) != 0) {  // (wave-uniform) a query block named more than once by one list
-        const float f0 = (float)w0, f1 = (float)w1;
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] *= r < 8 ? f0 : f1;
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      pb[r >> 3][r & 7] = (E)s[r];
-      db[r >> 3][r & 7] = (E)(s[r] * dp[r]);
-    }
+    staged_buf = -1;
   };
-  auto stage_c = [&](auto bufc, const int HF, const V8 (&pb)[2], const V8 (&db)[2]) {
-    constexpr int BUF = decltype(bufc)::value;
-    const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1) + HF * kHalfBytes;
-    const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1) + HF * kHalfBytes;
-    V8 gt[2][2], qt[2][2];
-    read_transposed<E>(gb, tr_off, gt);
-    read_transposed<E>(qb, tr_off, qt);
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-      for (int dt = 0; dt < 2; dt++) {
-        dvt[dt] = Mma<E>::mma(gt[jj][dt], pb[jj], dvt[dt]);
-        dkt[dt] = Mma<E>::mma(qt[jj][dt], db[jj], dkt[dt]);
-      }
-  };
-  // BLK 64: the same three stages with every instruction placed by hand, as in the forward kernel.  The vector work of
+  // One tile in three stages per 32-query half (A = row reads + S, dP; B = P and dS from the per-query scalars; C =
+  // transposed reads + dV^T, dK^T) with every instruction placed by hand, as in the forward kernel.  The vector work of
   // a 32-query half (16 scores per lane: P, dS, their roundings) is cut into eight slots of two scores; each slot also
   // issues one matrix product of another stage: the scores of half 1 run under the vector work of half 0, the dV / dK
   // products of half 0 under the vector work of half 1.  Only the scores of half 0 and the products of half 1 have no
@@ -832,6 +808,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     const char* qb = reinterpret_cast<const char*>(BUF == 0 ? lds_q0 : lds_q1);
     const char* gb = reinterpret_cast<const char*>(BUF == 0 ? lds_g0 : lds_g1);
     const float* sb = BUF == 0 ? lds_s0 : lds_s1;
+    const float* sl = sb + lse_at;  // BLK 16: the lse variant of this lane's key block
     f32x16 sc[2], dpv[2];   // S and dP of the two halves
     V8 pbv[2][2], dbv[2][2];  // P and dS as B operands [half][jj]
     V8 aq[4], ag[4];          // row fragments of Q, dO (A operands of the scores)
@@ -852,8 +829,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     auto vec = [&](auto hf_tag, auto j_tag) {  // scores 2j, 2j+1 of the half: P, dS, both rounded
       constexpr int HF = decltype(hf_tag)::value, j = decltype(j_tag)::value, r = 2 * j;
       // queries 4hh + 8(j/2) + 2(j%2) + {0, 1} of the half
-      const float2 l2 = *reinterpret_cast<const float2*>(sb + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
-      const float2 d2 = *reinterpret_cast<const float2*>(sb + 64 + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
+      const float2 l2 = *reinterpret_cast<const float2*>(sl + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
+      const float2 d2 = *reinterpret_cast<const float2*>(sl + kDeltaAt + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
       f32x16& sh = sc[HF];
       f32x16& dh = dpv[HF];
       const float p0 = __builtin_amdgcn_exp2f(fmaf(sh[r], sl2, -l2.x));
@@ -867,8 +844,19 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       dv[r & 7] = (E)e0;
       dv[(r & 7) + 1] = (E)e1;
     };
-    read_rows<E, true>(qb, c, hh, aq);
-    read_rows<E, true>(gb, c, hh, ag);
+    if constexpr (BLK == 64) {
+      read_rows<E, true>(qb, c, hh, aq);
+      read_rows<E, true>(gb, c, hh, ag);
+    } else {  // all eight fragments requested at once and waited for by hand: left to itself the compiler, short of
+      // registers further down the tile, reads them one at a time in this instance, each in front of its product
+      u32x4 qw[4], gw[4];
+      read_rows2_sync(qb, gb, c, hh, qw, gw);
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        aq[ks] = frag_of<E>(qw[ks]);
+        ag[ks] = frag_of<E>(gw[ks]);
+      }
+    }
     static_for<8>([&](auto i_tag) { mma_a(H0{}, i_tag); });
     __builtin_amdgcn_sched_barrier(0);
     // the fragments of a region's second four products are requested four slots ahead, one per slot, so that at most
@@ -889,29 +877,34 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       vec(H1{}, j_tag);
       __builtin_amdgcn_sched_barrier(0);
     });
-    read_transposed<E>(gb + kHalfBytes, tr_off, gt);
-    read_transposed<E>(qb + kHalfBytes, tr_off, qt);
-    static_for<8>([&](auto i_tag) { mma_c(H1{}, i_tag); });
-  };
-  auto compute_tile = [&](int64_t qblk, auto bufc) {
     if constexpr (BLK == 64) {
-      tile64(bufc);
-    } else {  // this wave's 32 keys against the 32 queries in its own half of the tile buffers
-      f32x16 s0, dp0;
-      V8 pb0[2], db0[2];
-      stage_a(bufc, wave, s0, dp0);
-      stage_b(qblk, bufc, wave, s0, dp0, pb0, db0);
-      stage_c(bufc, wave, pb0, db0);
+      read_transposed<E>(gb + kHalfBytes, tr_off, gt);
+      read_transposed<E>(qb + kHalfBytes, tr_off, qt);
+      static_for<8>([&](auto i_tag) { mma_c(H1{}, i_tag); });
+    } else {
+      u32x2 gw[2][2][2], qw[2][2][2];
+      read_transposed_sync(gb + kHalfBytes, tr_off, gw);
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) gt[jj][dt] = frag_of<E>(gw[jj][dt][0], gw[jj][dt][1]);
+      static_for<4>([&](auto i_tag) { mma_c(H1{}, i_tag); });
+      read_transposed_sync(qb + kHalfBytes, tr_off, qw);
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) qt[jj][dt] = frag_of<E>(qw[jj][dt][0], qw[jj][dt][1]);
+      static_for<4>([&](auto i_tag) { mma_c(H1{}, std::integral_constant<int, decltype(i_tag)::value + 4>{}); });
     }
   };
+  auto compute_tile = [&](int64_t qblk, auto bufc) { tile64(bufc); };
   // this wave's part of the tile has landed, its reads of the other buffer are done; after the barrier both hold
-  // for both waves (BLK 16: a wave only touches its own half of every buffer, so no barrier, and the two waves
-  // may walk lists of different lengths)
+  // for both waves
   auto sync = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     publish();
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    if constexpr (BLK == 64) __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_barrier();
   };
 
   auto walk = [&]() {  // all tiles of the current list, double buffered
@@ -940,181 +933,111 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
     store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
   } else {
-    // The wave holds TWO neighbouring key blocks A and B (32 different keys), whose lists name mostly the same query
-    // blocks (49 distinct ones for 2 x 32 entries at 266 496 tokens, top-32), and walks the UNION of the two lists, two
-    // distinct query blocks per step; every (query block, key block) quadrant of the 32 x 32 scores counts as often as
-    // that key block's list names the query block (0: not at all).  The union is built a chunk at a time: up to kChunk
-    // entries of list A, and the entries of list B below the first value A has left (both lists are ascending, so
-    // these are the entries that can meet this chunk of A), up to kChunk as well.  A chunk's entries go into a 512-slot
-    // hash table in an idle half of a tile buffer, by all lanes: compare-and-swap on the query block, linear probing, 1
-    // added to byte 0 (list A) or byte 1 (list B) of the slot's count; the occupied slots are compacted into lds_union,
-    // eight slots per lane, positions from ballots.  The steps come in the table's order (fp32 summation order only).
-    // Every list entry is in exactly one chunk, so whatever the chunks' borders, every (query block, key block) pair
-    // is counted as often as listed.  A pair of lists shared by the two waves (coop): wave 0 builds, both walk.
-    constexpr int kChunk = kMergeMax / 2;
-    int2* const uni = lds_union[BLK == 16 && !coop ? wave : 0];
-    int n_union = 0, step_no = 0, pa = 0, pb = 0;
-    auto build_chunk = [&]() -> bool {
-      const int na = len_a - pa < kChunk ? len_a - pa : kChunk;
-      const int32_t tau = pa + na < len_a ? __builtin_amdgcn_readfirstlane(lst_a[pa + na]) : 0x7fffffff;
-      int32_t bval[kChunk / 64];
-      int nb = 0;
+    // The workgroup's 64 keys are FOUR neighbouring key blocks, whose lists name mostly the same query blocks (at
+    // 266 496 tokens, top-32, the union of the four lists is half as long as the lists together), and the workgroup walks
+    // that union, four distinct query blocks per 64-row tile, with the 64-token kernel's tile code: a probability counts
+    // as often as its key block's list names its query block (`publish`).  The union is built a chunk at a time from
+    // the (ascending) lists: every list offers a window of its next kWin entries; tau = the smallest value that follows
+    // a window; the chunk takes the window entries below tau (the list that sets tau gives its whole window, so the
+    // walk advances; entries at or above tau may have partners in other lists that are not in their windows yet).
+    // Each wave inserts two of the lists into a 512-slot hash table in an idle tile buffer: compare-and-swap on the query
+    // block, linear probing, 1 added to the list's byte of the slot's count; wave 0 then compacts the occupied slots into
+    // lds_union, eight slots per lane, positions from ballots.  Tiles come in the table's order (fp32 summation order
+    // only).  Every list entry is in exactly one chunk, so whatever the chunks' borders, every (query block, key block)
+    // pair is counted as often as listed.
+    constexpr int kWin = kMergeMax / 4;
+    static_assert(kWin > 64 && kWin <= 128, "a window is read with two loads per lane; a query block repeats at most 64 times in a list");
+    const int64_t nkb16 = (Lk + 15) >> 4;
+    const int32_t* lp[4];
+    int llen[4], lpos[4];
 #pragma unroll
-      for (int jw = 0; jw < kChunk / 64; jw++) {
-        const int i = pb + 64 * jw + lane;
-        bval[jw] = i < len_b ? lst_b[i] : 0x7fffffff;
-        nb += __popcll(__ballot(bval[jw] < tau));  // a prefix of the window: the list is ascending
-      }
-      if (na + nb == 0) return false;
-      if (!coop || wave == 0) {
-        int32_t* const hkey = reinterpret_cast<int32_t*>(lds_q0 + wave * kHalfBytes);  // [512]
-        uint32_t* const hcnt = reinterpret_cast<uint32_t*>(lds_q0 + wave * kHalfBytes + 2048);  // [512]
-        reinterpret_cast<int4*>(hkey)[lane] = make_int4(-1, -1, -1, -1);
-        reinterpret_cast<int4*>(hkey)[lane + 64] = make_int4(-1, -1, -1, -1);
-        reinterpret_cast<int4*>(hcnt)[lane] = make_int4(0, 0, 0, 0);
-        reinterpret_cast<int4*>(hcnt)[lane + 64] = make_int4(0, 0, 0, 0);
-        auto insert = [&](bool active, int32_t e, uint32_t one) {
-          uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
-          while (active) {
-            const int32_t old = atomicCAS(hkey + slot, -1, e);
-            if (old == -1 || old == e) {
-              atomicAdd(hcnt + slot, one);
-              active = false;
-            } else {
-              slot = (slot + 1) & 511u;
-            }
-          }
-        };
-#pragma unroll
-        for (int jw = 0; jw < kChunk / 64; jw++) {
-          const int i = 64 * jw + lane;
-          const bool act = i < na;
-          insert(act, act ? lst_a[pa + i] : 0, 1u);
+    for (int i4 = 0; i4 < 4; i4++) {
+      const int64_t kblk = (int64_t)kb * 4 + i4;
+      const bool there = kblk < nkb16;
+      const int32_t o0 = there ? __builtin_amdgcn_readfirstlane(off16[kblk]) : 0;
+      const int32_t o1 = there ? __builtin_amdgcn_readfirstlane(off16[kblk + 1]) : 0;
+      lp[i4] = list + o0;
+      llen[i4] = o1 - o0;
+      lpos[i4] = 0;
+    }
+    int32_t* const hkey = reinterpret_cast<int32_t*>(lds_q0);          // [512]
+    uint32_t* const hcnt = reinterpret_cast<uint32_t*>(lds_q0 + 2048);  // [512]
+    auto insert = [&](bool active, int32_t e, uint32_t one) {
+      uint32_t slot = ((uint32_t)e * 0x9E3779B1u) >> 23;
+      while (active) {
+        const int32_t old = atomicCAS(hkey + slot, -1, e);
+        if (old == -1 || old == e) {
+          atomicAdd(hcnt + slot, one);
+          active = false;
+        } else {
+          slot = (slot + 1) & 511u;
         }
+      }
+    };
+    auto build_chunk = [&]() -> bool {  // false: the lists are exhausted.  Both waves take the same decisions.
+      // all eight loads in one round trip: lane kWin - 64 of a list's second load fetches the value after the window
+      int32_t ev[4][2];
 #pragma unroll
-        for (int jw = 0; jw < kChunk / 64; jw++) insert(64 * jw + lane < nb, bval[jw], 256u);
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int i0 = lpos[i4] + lane, i1 = lpos[i4] + 64 + lane;
+        ev[i4][0] = i0 < llen[i4] ? lp[i4][i0] : 0x7fffffff;
+        ev[i4][1] = lane <= kWin - 64 && i1 < llen[i4] ? lp[i4][i1] : 0x7fffffff;
+      }
+      int32_t tau = 0x7fffffff;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int32_t nextv = __builtin_amdgcn_readlane(ev[i4][1], kWin - 64);
+        tau = nextv < tau ? nextv : tau;
+        if (lane == kWin - 64) ev[i4][1] = 0x7fffffff;  // not part of the window
+      }
+      int taken[4], total = 0;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        taken[i4] = __popcll(__ballot(ev[i4][0] < tau)) + __popcll(__ballot(ev[i4][1] < tau));  // a prefix: the list is ascending
+        total += taken[i4];
+      }
+      if (total == 0) return false;
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): this wave is through the previous chunk's tiles
+      __syncthreads();                      // ... and so is the other one: the table's buffer and the list are free
+      reinterpret_cast<int4*>(hkey)[threadIdx.x] = make_int4(-1, -1, -1, -1);
+      reinterpret_cast<int4*>(hcnt)[threadIdx.x] = make_int4(0, 0, 0, 0);
+      __syncthreads();
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        if ((i4 >> 1) == wave) {  // (wave-uniform) this wave's two lists
+          insert(ev[i4][0] < tau, ev[i4][0], 1u << (8 * i4));
+          insert(ev[i4][1] < tau, ev[i4][1], 1u << (8 * i4));
+        }
+        lpos[i4] += taken[i4];
+      }
+      __syncthreads();
+      if (wave == 0) {
         const int4 k0 = reinterpret_cast<const int4*>(hkey)[2 * lane], k1 = reinterpret_cast<const int4*>(hkey)[2 * lane + 1];
         const int4 c0 = reinterpret_cast<const int4*>(hcnt)[2 * lane], c1 = reinterpret_cast<const int4*>(hcnt)[2 * lane + 1];
         const int32_t ks8[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
         const int32_t cs8[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-        uint32_t pos = 0;  // occupied slots of the lanes below
-        n_union = 0;
+        uint32_t at = 0;  // occupied slots of the lanes below
+        int n_union = 0;
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
           const uint64_t m = __ballot(ks8[s8] >= 0);
-          pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, pos));
+          at = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, at));
           n_union += __popcll(m);
         }
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++)
-          if (ks8[s8] >= 0) uni[pos++] = make_int2(ks8[s8], cs8[s8]);
-        if (lane == 0) {
-          uni[n_union] = make_int2(-1, 0);      // the partner of an odd last entry
-          uni[kMergeMax + 1] = make_int2(n_union, 0);  // for the other wave of a shared pair
-        }
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): table read, list written before the first transfer lands there
-      }
-      pa += na;
-      pb += nb;
-      if (coop) {
-        __syncthreads();
-        n_union = __builtin_amdgcn_readfirstlane(uni[kMergeMax + 1].x);
-      }
-      step_no = 0;
-      return true;
-    };
-    // The next step of this wave: entries 2t, 2t + 1 of the chunk's union as two query blocks (packed for `fetch`; -1:
-    // none) and their four weights, byte 2 * entry + key block.  A shared pair: the two waves take alternate steps.
-    auto next_step = [&](int64_t& blocks, uint32_t& w) -> bool {
-      const int t = coop ? 2 * step_no + wave : step_no;
-      step_no++;
-      if (2 * t >= n_union) return false;
-      const int4 v = *reinterpret_cast<const int4*>(uni + 2 * t);
-      const int32_t q0 = __builtin_amdgcn_readfirstlane(v.x), q1 = __builtin_amdgcn_readfirstlane(v.z);
-      const uint32_t c0 = (uint32_t)__builtin_amdgcn_readfirstlane(v.y), c1 = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
-      w = (c0 & 0xffffu) | (c1 << 16);
-      blocks = (int64_t)(uint32_t)q0 | ((int64_t)q1 << 32);
-      return true;
-    };
-    auto walk16 = [&]() {  // all steps of the current chunk, double buffered
-      int64_t cur = 0, nxt = 0;
-      uint32_t wcur = 0, wnxt = 0;
-      if (!next_step(cur, wcur)) return;
-      fetch(cur, H0{});
-      while (true) {
-        sync();
-        const bool more1 = next_step(nxt, wnxt);
-        if (more1) fetch(nxt, H1{});
-        step_w = wcur;
-        compute_tile(cur, H0{});
-        if (!more1) break;
-        sync();
-        const bool more2 = next_step(cur, wcur);
-        if (more2) fetch(cur, H0{});
-        step_w = wnxt;
-        compute_tile(nxt, H1{});
-        if (!more2) break;
-      }
-    };
-    // Workgroups of the long-list pass: both waves walk each of the tile's two pairs of key blocks together (alternate
-    // steps), so a long list is shared and the two waves stay in balance; at the end of a pair the second wave hands its
-    // partial sums over through LDS (the tile buffers are idle then).  Otherwise each wave takes its own pair.
-    const int64_t nkb16 = (Lk + 15) >> 4;
-    for (int li = 0; li < (coop ? 2 : 1); li++) {
-      const int64_t kblk = (int64_t)kb * 4 + 2 * (coop ? li : wave);  // key block A; B = A + 1 (may not exist)
-      if (kblk * 16 >= Lk) break;  // no such key blocks (shared pairs: the same for both waves)
-      key = kblk * 16 + c;
-      const int32_t oa = __builtin_amdgcn_readfirstlane(off16[kblk]), ob = __builtin_amdgcn_readfirstlane(off16[kblk + 1]);
-      lst_a = list + oa;
-      len_a = ob - oa;
-      lst_b = list + ob;
-      len_b = kblk + 1 < nkb16 ? __builtin_amdgcn_readfirstlane(off16[kblk + 2]) - ob : 0;
-      pa = pb = 0;
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's last LDS reads are done before new transfers land
-      load_keys();
-      while (build_chunk()) {
-        walk16();
-        if (coop) {
-          __builtin_amdgcn_s_waitcnt(0xC07F);
-          __syncthreads();  // both waves are through the chunk before its list and the table's buffer are reused
-        }
-      }
-      const bool live = key < Lk;
-      if (!coop) {
-        store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
-        store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
-        continue;
-      }
-      // wave 1 -> wave 0: 64 values per lane, value i of lane l at float i * 64 + l of the four tile buffers
-      auto slot = [&](int i) -> float* {
-        unsigned char* a = i < 32 ? (i < 16 ? lds_q0 : lds_q1) : (i < 48 ? lds_g0 : lds_g1);
-        return reinterpret_cast<float*>(a) + (i & 15) * 64 + lane;
-      };
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): none of this wave's transfers is still writing the buffers
-      __syncthreads();                      // both waves are done with the tile buffers
-      if (wave == 1) {
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            *slot(dt * 16 + r) = dkt[dt][r];
-            *slot(32 + dt * 16 + r) = dvt[dt][r];
-          }
+          if (ks8[s8] >= 0) lds_union[at++] = make_int2(ks8[s8], cs8[s8]);
+        if (lane < 4) lds_union[n_union + lane] = make_int2(-1, 0);  // the last tile's missing entries
+        if (lane == 0) lds_union[kMergeMax + 7] = make_int2(n_union, 0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the table is read before the first transfer lands on it
       }
       __syncthreads();
-      if (wave == 0) {
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            dkt[dt][r] += *slot(dt * 16 + r);
-            dvt[dt][r] += *slot(32 + dt * 16 + r);
-          }
-        store_rows<E>(dkt, dkp + key * p.sdkn, live, hh);
-        store_rows<E>(dvt, dvp + key * p.sdvn, live, hh);
-      }
-      __syncthreads();  // the hand-over is read before the next list's transfers overwrite it
-    }
+      n_lists = (__builtin_amdgcn_readfirstlane(lds_union[kMergeMax + 7].x) + 3) >> 2;  // tiles of this chunk
+      return true;
+    };
+    while (build_chunk()) walk();
+    store_rows<E>(dkt, dkp + key * p.sdkn, key < Lk, hh);
+    store_rows<E>(dvt, dvp + key * p.sdvn, key < Lk, hh);
   }
 }
 

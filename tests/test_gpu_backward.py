@@ -121,9 +121,8 @@ def test_selection_backward_with_16_token_blocks_skips_duplicates_and_popular_ke
 
 @pytest.mark.parametrize("n,kk", [(1040, 2), (2000, 4), (650, 1)])
 def test_selection_backward_with_16_token_blocks_and_very_long_lists(n, kk):
-    """Key blocks that nearly every query block lists: their tiles take the path in which the two waves of a
-    workgroup share each list and hand partial sums over through LDS (lists much longer than 4 * top-k), next to
-    ordinary tiles and a ragged last block."""
+    """Key blocks that nearly every query block lists: the union of their workgroup's four lists is built in several
+    chunks (a list offers 96 entries per chunk), next to ordinary tiles and a ragged last block."""
     b, h = 1, 2
     nqb = -(-n // 16)
     q, k, v, g = (_randn((b, h, n, 64), 170 + i, torch.bfloat16, 0.5 if i < 3 else 1.0) for i in range(4))
@@ -131,6 +130,29 @@ def test_selection_backward_with_16_token_blocks_and_very_long_lists(n, kk):
     idx[0, 0, :, 0] = 9                        # on every list of head 0
     idx[0, 1, ::2, 0] = nqb - 1                # the ragged last block on every second list of head 1
     idx[0, 1, 1::2, 0] = 3
+    qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
+    o, lse = s3r.select_attn(qd, kd, vd, idxd, 16, return_lse=True)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd, 16)
+    mult = oracle.block_multiplicity(idx, n, 16)
+    wq, wk, wv, _, _ = oracle.attention_grads_formula(q, k, v, g, mult)
+    _close(dq, wq, "dq"); _close(dk, wk, "dk"); _close(dv, wv, "dv")
+
+
+def test_selection_backward_with_16_token_blocks_and_long_lists_side_by_side():
+    """Four neighbouring key blocks of one workgroup with long lists of different lengths (all, every second, every
+    third query block, a run in the middle), one of them named twice by some query blocks: every chunk of the union
+    takes entries from several lists, and the chunk borders fall differently in each."""
+    b, h, n, kk = 1, 2, 4000, 6
+    nqb = n // 16
+    q, k, v, g = (_randn((b, h, n, 64), 190 + i, torch.bfloat16, 0.5 if i < 3 else 1.0) for i in range(4))
+    idx = _rand_idx(b, h, nqb, kk, nqb, 195)
+    idx[0, 0, :, 0] = 8                        # key blocks 8..11 are one workgroup's
+    idx[0, 0, ::2, 1] = 9
+    idx[0, 0, ::3, 2] = 10
+    idx[0, 0, 60:200, 3] = 11
+    idx[0, 0, 100:130, 4] = 8                  # ... and 8 twice on these lists
+    idx[0, 1, :, 0] = 41                       # head 1: two long lists in different workgroups' neighbourhoods
+    idx[0, 1, 5:, 1] = 43
     qd, kd, vd, gd, idxd = (t.to(DEV) for t in (q, k, v, g, idx))
     o, lse = s3r.select_attn(qd, kd, vd, idxd, 16, return_lse=True)
     dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, gd, lse, idxd, 16)
