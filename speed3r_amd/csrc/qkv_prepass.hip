@@ -20,7 +20,9 @@ namespace s3r {
 // at a time and q's temporaries are dead before k's are born: the kernel lives on many resident waves (128 registers,
 // four per SIMD), not on deep batches per wave -- with two steps in flight the register file held half as many waves
 // and the pass took 2.4 times as long.
-template <typename T>
+// ALL: LayerNorm with bias and positions are all there (the layer's own call): their run-time tests, and the default
+// values of the paths not taken, are then not compiled in.
+template <typename T, bool ALL>
 __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ q_out, T* __restrict__ k_out,
     T* __restrict__ qc, T* __restrict__ kc, T* __restrict__ vc, const int32_t* __restrict__ pos, const T* __restrict__ cos_tab,
@@ -55,7 +57,8 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
 
   // LayerNorm parameters of the lane's 16 bytes (q_norm and k_norm are different modules): fetched in every step from
   // the vector cache rather than held, their 16 registers are worth more as room for one more resident wave
-  const bool norm = qn_w != nullptr;
+  const bool norm = ALL || qn_w != nullptr;
+  const bool rotate = ALL || pos != nullptr;
   // The block's positions, fetched with two coalesced loads per 64 tokens (lane l holds values l and 64 + l of the
   // (y, x) pairs) and handed out by shuffles: the table rows of a step then need no load of their own position first.
   int pos_lo = 0, pos_hi = 0;
@@ -70,23 +73,32 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
 #pragma unroll
   for (int i = 0; i < VEC; i++) aq[i] = ak[i] = av[i] = 0.f;
 
-  for (int rbase = 0; rbase < nvalid; rbase += RPW) {  // wave-uniform trip count: the position shuffles span the wave
+  // one wave-wide step; WHOLE: all its rows are inside the block (no row to keep out of the sums and the stores)
+  auto step = [&](int rbase, auto whole_tag) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
     const int rr = rbase + r0;
-    const bool keep = rr < nvalid;
+    const bool keep = WHOLE || rr < nvalid;
     const int rcl = keep ? rr : nvalid - 1;  // rows beyond the block shadow its last row (not added, not stored)
-    if (pos != nullptr && (rbase & 63) == 0) fetch_positions(rbase);
+    if (rotate && (rbase & 63) == 0) fetch_positions(rbase);
     const int64_t off = in_off + (t0 + rcl) * sxn;
     const u32x4 lq = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + off));
     const u32x4 lk = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k + off));
     const u32x4 lv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(v + off));
     uint4 rc = make_uint4(0, 0, 0, 0), rs = rc;
-    if (pos != nullptr) {
+    if (rotate) {
       const int slot = 2 * (rcl & 63) + half;  // index of (token, y or x) among the fetched 128
       const int from_lo = __shfl(pos_lo, slot & 63), from_hi = __shfl(pos_hi, slot & 63);
       int pp = slot < 64 ? from_lo : from_hi;
       pp = pp < 0 ? 0 : (pp >= P ? P - 1 : pp);
       rc = *reinterpret_cast<const uint4*>(cos_tab + (int64_t)pp * (D / 4) + f0);
       rs = *reinterpret_cast<const uint4*>(sin_tab + (int64_t)pp * (D / 4) + f0);
+      if constexpr (sizeof(T) == 2) {
+        // "rotate half" is (-second quarter, first quarter): the lanes of a first quarter take their partner's value
+        // with a minus sign, which is put on the sine instead, on the packed words (rounding is symmetric:
+        // round(-a * s) = round(a * -s), the same bits)
+        const uint32_t flip = second ? 0u : 0x80008000u;
+        rs.x ^= flip; rs.y ^= flip; rs.z ^= flip; rs.w ^= flip;
+      }
     }
     const T* ce = reinterpret_cast<const T*>(&rc);
     const T* se = reinterpret_cast<const T*>(&rs);
@@ -96,7 +108,7 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
       uint4 wgt_raw = make_uint4(0, 0, 0, 0), bias_raw = wgt_raw;
       if (norm) {
         wgt_raw = *reinterpret_cast<const uint4*>(ln_w + lr * VEC);
-        if (ln_b != nullptr) bias_raw = *reinterpret_cast<const uint4*>(ln_b + lr * VEC);
+        if (ALL || ln_b != nullptr) bias_raw = *reinterpret_cast<const uint4*>(ln_b + lr * VEC);
       }
       const T* wgt = reinterpret_cast<const T*>(&wgt_raw);
       const T* bias = reinterpret_cast<const T*>(&bias_raw);
@@ -120,11 +132,11 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
 #pragma unroll
         for (int i = 0; i < VEC; i++) x[i] = round_to<T>((x[i] - mean) * rstd * to_f32(wgt[i]) + to_f32(bias[i]));
       }
-      if (pos != nullptr) {
+      if (rotate) {
 #pragma unroll
         for (int i = 0; i < VEC; i++) {
           const float other = lane_xor<QL>(x[i]);     // the paired value, one quarter away
-          const float rot = second ? other : -other;  // "rotate half": (-second quarter, first quarter)
+          const float rot = sizeof(T) == 2 || second ? other : -other;  // (16-bit types: the sign is on the sine)
           const float a = round_to<T>(x[i] * to_f32(ce[i]));
           const float c2 = round_to<T>(rot * to_f32(se[i]));
           x[i] = a + c2;
@@ -140,6 +152,10 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
     one(lq, aq, qn_w, qn_b, qo);
     __builtin_amdgcn_sched_barrier(0);  // q's temporaries are dead before k's are born
     one(lk, ak, kn_w, kn_b, ko);
+  };
+  for (int rbase = 0; rbase < nvalid; rbase += RPW) {  // wave-uniform trip count: the position shuffles span the wave
+    if (rbase + RPW <= nvalid) step(rbase, std::true_type{});
+    else step(rbase, std::false_type{});
   }
   // block means: fold the row groups, divide by the number of valid tokens
   for (int off = LPR; off < 64; off <<= 1) {
@@ -191,13 +207,20 @@ extern "C" int s3r_qkv_prepass(const void* q, const void* k, const void* v, void
   if (blocks > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_qkv_prepass: tensor too large for one launch");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)blocks), blk(256);
-#define S3R_PREPASS(T)                                                                                                              \
-  hipLaunchKernelGGL(qkv_prepass_kernel<T>, grid, blk, 0, st, (const T*)q, (const T*)k, (const T*)v, (T*)q_out, (T*)k_out, (T*)qc, \
-                     (T*)kc, (T*)vc, pos, (const T*)cos_tab, (const T*)sin_tab, P, (const T*)qn_w, (const T*)qn_b, (const T*)kn_w,  \
-                     (const T*)kn_b, eps, H, N, block, Nc, total, sxb, sxh, sxn, spb, spn)
+  const bool all = pos != nullptr && qn_w != nullptr && qn_b != nullptr && kn_b != nullptr;
+#define S3R_PREPASS_ARGS(T)                                                                                                       \
+  grid, blk, 0, st, (const T*)q, (const T*)k, (const T*)v, (T*)q_out, (T*)k_out, (T*)qc, (T*)kc, (T*)vc, pos, (const T*)cos_tab,  \
+      (const T*)sin_tab, P, (const T*)qn_w, (const T*)qn_b, (const T*)kn_w, (const T*)kn_b, eps, H, N, block, Nc, total, sxb, sxh, \
+      sxn, spb, spn
+#define S3R_PREPASS(T)                                                                   \
+  do {                                                                                   \
+    if (all) hipLaunchKernelGGL((qkv_prepass_kernel<T, true>), S3R_PREPASS_ARGS(T));     \
+    else hipLaunchKernelGGL((qkv_prepass_kernel<T, false>), S3R_PREPASS_ARGS(T));        \
+  } while (0)
   if (dtype == S3R_F32) S3R_PREPASS(float);
   else if (dtype == S3R_BF16) S3R_PREPASS(bf16_t);
   else S3R_PREPASS(f16_t);
 #undef S3R_PREPASS
+#undef S3R_PREPASS_ARGS
   return check_launch("s3r_qkv_prepass");
 }
