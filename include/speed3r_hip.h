@@ -262,7 +262,8 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
  *   kq_list, kq_off (needed for dk/dv when idx is given): for every (b,h) the query-block ids that list key block j,
  *     one entry per occurrence, ascending, are kq_list[(b*H+h)*list_stride + kq_off[(b*H+h)*(nkb+1) + j] ...
  *     kq_off[... + j+1]), nkb = ceil(Lk/block); entries of idx that are < 0 or >= nkb appear in no list
- *     (reference count_query_fixedlen / reorder_topk_idx_fixedlen, :423-554).
+ *     (reference count_query_fixedlen / reorder_topk_idx_fixedlen, :423-554).  With block 16 the dk/dv kernel merges
+ *     neighbouring lists and relies on every list being ascending, as s3r_key_block_lists leaves it.
  *   dq (layout strides sdq*), dk, dv (sdk*, sdv*): I/O dtype; dq == NULL or dk == dv == NULL skips that kernel.
  *   Every row of dq, dk, dv inside the tensors is written (zeros where nothing attends).
  */
