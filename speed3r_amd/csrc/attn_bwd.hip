@@ -897,7 +897,6 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       static_for<4>([&](auto i_tag) { mma_c(H1{}, std::integral_constant<int, decltype(i_tag)::value + 4>{}); });
     }
   };
-  auto compute_tile = [&](int64_t qblk, auto bufc) { tile64(bufc); };
   // this wave's part of the tile has landed, its reads of the other buffer are done; after the barrier both hold
   // for both waves
   auto sync = [&]() {
@@ -916,13 +915,13 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
         const bool more1 = t + 1 < n_lists;
         const int64_t nxt1 = more1 ? block_of(t + 1) : cur;
         if (more1) fetch(nxt1, H1{});
-        compute_tile(cur, H0{});
+        tile64(H0{});
         if (!more1) break;
         sync();
         const bool more2 = t + 2 < n_lists;
         cur = more2 ? block_of(t + 2) : nxt1;
         if (more2) fetch(cur, H0{});
-        compute_tile(nxt1, H1{});
+        tile64(H1{});
       }
     }
   };
