@@ -386,6 +386,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 #pragma unroll
     for (int s8 = 0; s8 < 8; s8++)
       if (ks8[s8] >= 0) walk[pos++] = make_int2(ks8[s8], cs8[s8]);
+    if (lane < 4) walk[n_union + lane] = make_int2(-1, 0);  // the last tile's missing entries
     dup = __any((cnt_bits & 0xfefefefeu) != 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the table is read and the list written before the first transfer
     ntiles = (n_union + 3) >> 2;
@@ -401,17 +402,26 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       return (int64_t)(dense_next++);
     }
   };
-  // BLK 16: first key row, number of valid rows and the four count bytes of entry `s` (0..3) of tile t of the walk
-  // list (past the list's end: row 0, no counts)
-  auto sub_block = [&](int64_t t, int s, int64_t& start, int& nv, uint32_t& counts) {
-    const int e = 4 * (int)t + s;
-    u32x2 v = {0xffffffffu, 0u};
-    if (e < n_union) {  // (wave-uniform) a hand-written read, like the fragments'
-      const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)reinterpret_cast<const char*>(walk + e);
-      asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a));
-    }
-    const int32_t blk = __builtin_amdgcn_readfirstlane((int32_t)v[0]);
-    counts = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v[1]);
+  // BLK 16: the four entries (key block, four count bytes; -1: none) of the tile being computed and of the tile whose
+  // first half is fetched meanwhile, read from the walk list once per tile (a hand-written read, like the fragments')
+  // and kept in scalar registers
+  struct Entries16 { int32_t blk[4] = {-1, -1, -1, -1}; uint32_t cnt[4] = {0, 0, 0, 0}; };
+  struct NoEntries {};
+  typedef std::conditional_t<BLK == 16, Entries16, NoEntries> TileEntries;
+  TileEntries ent_cur, ent_nxt;
+  auto read_entries = [&](int64_t t, Entries16& e) {
+    const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)reinterpret_cast<const char*>(walk + 4 * t);
+    u32x4 v0, v1;
+    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:16\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v0), "=&v"(v1) : "v"(a));
+    e.blk[0] = __builtin_amdgcn_readfirstlane((int32_t)v0[0]); e.cnt[0] = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v0[1]);
+    e.blk[1] = __builtin_amdgcn_readfirstlane((int32_t)v0[2]); e.cnt[1] = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v0[3]);
+    e.blk[2] = __builtin_amdgcn_readfirstlane((int32_t)v1[0]); e.cnt[2] = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v1[1]);
+    e.blk[3] = __builtin_amdgcn_readfirstlane((int32_t)v1[2]); e.cnt[3] = (uint32_t)__builtin_amdgcn_readfirstlane((int32_t)v1[3]);
+  };
+  // first key row, number of valid rows and the count bytes of entry `s` (0..3) of a tile (none: row 0, no counts)
+  auto sub_block = [&](const Entries16& e, int s, int64_t& start, int& nv, uint32_t& counts) {
+    const int32_t blk = e.blk[s];
+    counts = e.cnt[s];
     start = blk >= 0 ? (int64_t)blk * 16 : 0;
     nv = blk >= 0 ? (int)(Lk - start < 16 ? Lk - start : 16) : 0;
   };
@@ -421,7 +431,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
   const uint32_t krow = (uint32_t)p.skn * (uint32_t)sizeof(E), vrow = (uint32_t)p.svn * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
 
-  auto fetch = [&](int64_t start, auto hf, int buf) {  // half HF of the tile at `start` -> buffers `buf`
+  auto fetch = [&](int64_t start, auto hf, int buf, const TileEntries& ent) {  // half HF of the tile at `start` -> buffers `buf`
     constexpr int HF = decltype(hf)::value;
     if constexpr (BLK == 64) {
       const int last = (int)((Lk - start < 64 ? Lk - start : 64) - 1);
@@ -431,14 +441,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       int64_t sa, sb;
       int na, nb;
       uint32_t ca, cb;
-      sub_block(start, 2 * HF, sa, na, ca);
-      sub_block(start, 2 * HF + 1, sb, nb, cb);
+      sub_block(ent, 2 * HF, sa, na, ca);
+      sub_block(ent, 2 * HF + 1, sb, nb, cb);
       const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
       dma_rows16<E, true>(kp + sa * p.skn, kp + sb * p.skn, krow, la, lb, k_buf[buf], lane);
       dma_rows16<E, false>(vp + sa * p.svn, vp + sb * p.svn, vrow, la, lb, v_buf[buf], lane);
     }
   };
-  auto compute = [&](int64_t start, auto hf, int buf) {
+  auto compute = [&](int64_t start, auto hf, int buf, const TileEntries& ent) {
     constexpr int HF = decltype(hf)::value;
     int nvalid = 64;
     int na = 16, nb = 16;      // BLK 16: valid keys of the half's two blocks A (rows 0..15) and B (16..31)
@@ -447,8 +457,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       nvalid = (int)(Lk - start < 64 ? Lk - start : 64);
     } else {
       int64_t sa, sb;
-      sub_block(start, 2 * HF, sa, na, ca);
-      sub_block(start, 2 * HF + 1, sb, nb, cb);
+      sub_block(ent, 2 * HF, sa, na, ca);
+      sub_block(ent, 2 * HF + 1, sb, nb, cb);
     }
     const bool ragged = nvalid < 64;
     V8 ak[4], av[4];
@@ -472,26 +482,31 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
       for (int ks = 0; ks < 4; ks++) st = Mma<E>::mma(ak[ks], bq[qt][ks], st);
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) dp = Mma<E>::mma(av[ks], bg[qt][ks], dp);
-#pragma unroll
-      for (int r = 0; r < 16; r++) st[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));  // P^T
       if constexpr (BLK == 64) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) st[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -lse2[qt]));  // P^T
         if (ragged) {  // keys beyond Lk carry no probability
 #pragma unroll
           for (int r = 0; r < 16; r++)
             if (32 * HF + 4 * hh + 8 * (r >> 2) + (r & 3) >= nvalid) st[r] = 0.f;
         }
-      } else {  // registers 0..7 are keys of block A, 8..15 of block B; this lane's query block lists each 0, 1 or more times
+      } else {
+        // registers 0..7 are keys of block A, 8..15 of block B; this lane's query block lists each 0, 1 or more times,
+        // and a probability counts that often: the count goes into the exponent (lse - log2(count); 0 times: +inf),
+        // two values per lane instead of a test per score
         const int sh = 8 * (2 * qt + (c >> 4));
         const uint32_t wa = (ca >> sh) & 0xffu, wb = (cb >> sh) & 0xffu;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const bool on = (r < 8 ? wa : wb) != 0 && 4 * hh + 8 * ((r >> 2) & 1) + (r & 3) < (r < 8 ? na : nb);
-          st[r] = on ? st[r] : 0.f;
-        }
+        float la = wa != 0 ? lse2[qt] : INFINITY, lb = wb != 0 ? lse2[qt] : INFINITY;
         if (dup) {
-          const float fa = (float)wa, fb = (float)wb;
+          la -= __builtin_amdgcn_logf((float)(wa > 1 ? wa : 1));
+          lb -= __builtin_amdgcn_logf((float)(wb > 1 ? wb : 1));
+        }
 #pragma unroll
-          for (int r = 0; r < 16; r++) st[r] *= r < 8 ? fa : fb;
+        for (int r = 0; r < 16; r++) st[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, -(r < 8 ? la : lb)));  // P^T
+        if (na < 16 || nb < 16) {  // (wave-uniform) a block cut short by the end of the sequence, or none
+#pragma unroll
+          for (int r = 0; r < 16; r++)
+            if (4 * hh + 8 * ((r >> 2) & 1) + (r & 3) >= (r < 8 ? na : nb)) st[r] = 0.f;
         }
       }
 #pragma unroll
@@ -516,23 +531,28 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdParams p, int nqb, in
 
   if (ntiles > 0) {
     int64_t cur = pop();
-    fetch(cur, H0{}, 0);
+    if constexpr (BLK == 16) read_entries(cur, ent_cur);
+    fetch(cur, H0{}, 0, ent_cur);
     for (int t = 0; t < ntiles; t++) {
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffer 1 (previous tile) are done
-      fetch(cur, H1{}, 1);
+      fetch(cur, H1{}, 1, ent_cur);
       __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): half 0 has landed
-      compute(cur, H0{}, 0);
+      compute(cur, H0{}, 0, ent_cur);
       const bool more = t + 1 < ntiles;
       const int64_t nxt = more ? pop() : cur;
+      if constexpr (BLK == 16) {
+        if (more) read_entries(nxt, ent_nxt);
+      }
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the reads of buffer 0 are done
       if (more) {
-        fetch(nxt, H0{}, 0);
+        fetch(nxt, H0{}, 0, ent_nxt);
         __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): half 1 has landed
       } else {
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       }
-      compute(cur, H1{}, 1);
+      compute(cur, H1{}, 1, ent_cur);
       cur = nxt;
+      ent_cur = ent_nxt;
     }
   }
 
