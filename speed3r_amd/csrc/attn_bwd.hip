@@ -756,31 +756,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       const int na = ea >= 0 ? (int)(Lq - sa < 16 ? Lq - sa : 16) : 0;
       const int nb = eb >= 0 ? (int)(Lq - sbk < 16 ? Lq - sbk : 16) : 0;
       const int la = na > 0 ? na - 1 : 0, lb = nb > 0 ? nb - 1 : 0;
-      if (na == 16 && nb == 16) {
-        // (wave-uniform) two full blocks: the per-lane offsets of a full tile serve (the chunk map ignores row bit 4),
-        // rows 8..15 of a block ride in the scalar offset
-        const __amdgpu_buffer_rsrc_t rqa = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + sa * p.sqm), 0, 0x7fffffff, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rqb = __builtin_amdgcn_make_buffer_rsrc((void*)(qp + sbk * p.sqm), 0, 0x7fffffff, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rga = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + sa * p.sgm), 0, 0x7fffffff, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rgb = __builtin_amdgcn_make_buffer_rsrc((void*)(gp + sbk * p.sgm), 0, 0x7fffffff, 0x00020000);
-        char* qh = qb + wave * kHalfBytes;
-        char* gh = gb + wave * kHalfBytes;
-        // the per-lane offsets are made here, from a copy of the lane number the compiler cannot see through: kept
-        // across the tile's work they would cost the four registers that the tile code has not got
-        int ln = lane;
-        asm volatile("" : "+v"(ln));
-        const uint32_t ch[2] = {(uint32_t)(((ln & 7) ^ k_swizzle(ln >> 3)) * 16), (uint32_t)(((ln & 7) ^ k_swizzle((ln >> 3) + 8)) * 16)};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? rqa : rqb, (__attribute__((address_space(3))) void*)(qh + i * 1024), 16,
-                                                   (uint32_t)(ln >> 3) * qrow + ch[i & 1], (i & 1) * 8 * qrow, 0, 0);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(i < 2 ? rga : rgb, (__attribute__((address_space(3))) void*)(gh + i * 1024), 16,
-                                                   (uint32_t)(ln >> 3) * grow + ch[i & 1], (i & 1) * 8 * grow, 0, 0);
-        }
-      } else {
-        dma_rows16<E, true>(qp + sa * p.sqm, qp + sbk * p.sqm, qrow, la, lb, qb + wave * kHalfBytes, lane);
-        dma_rows16<E, true>(gp + sa * p.sgm, gp + sbk * p.sgm, grow, la, lb, gb + wave * kHalfBytes, lane);
-      }
+      dma_rows16<E, true>(qp + sa * p.sqm, qp + sbk * p.sqm, qrow, la, lb, qb + wave * kHalfBytes, lane);
+      dma_rows16<E, true>(gp + sa * p.sgm, gp + sbk * p.sgm, grow, la, lb, gb + wave * kHalfBytes, lane);
       const int j = lane & 31, j16 = j & 15;
       const bool second = (j >> 4) != 0;
       const int nmine = second ? nb : na;
