@@ -669,8 +669,12 @@ int launch_select_pipe(const AttnParams& p, int dtype, void* stream) {
   const int64_t nqb = (p.Lq + 63) / 64;
   const bool dense = p.idx == nullptr;  // no index list: every query block sweeps all key tiles
   if (dense && p.Lq != p.Lk) return fail(S3R_ERR_UNSUPPORTED, "dense sweep: Lq %lld != Lk %lld", (long long)p.Lq, (long long)p.Lk);
-  // a dense sweep with fewer waves than 1.5 per SIMD of the chip (256 CUs x 4) runs with two waves per query block
-  const bool split = dense && nqb * p.B * p.H < 1536;
+  // A dense sweep runs with two waves per query block where it has fewer waves than 1.5 per SIMD of the chip (256 CUs x
+  // 4), and where its waves fill the chip's 2048 places (two per SIMD) a whole number of times plus a small rest: the
+  // rest runs as a round of its own, and with half the key tiles per wave that round is half as long (16 656 pooled
+  // tokens x 16 heads = 4176 waves: 1.27 -> 1.21 ms; without such a rest the split costs 2 %).
+  const int64_t sweeps = nqb * p.B * p.H;
+  const bool split = dense && (sweeps < 1536 || (sweeps > 2048 && sweeps % 2048 != 0 && (sweeps % 2048) * 5 < 2048));
   const int per_wg = split ? pipe::kWaves / 2 : pipe::kWaves;
   const int64_t nqg = (nqb + per_wg - 1) / per_wg;
   const int64_t total = nqg * p.B * p.H;

@@ -118,12 +118,13 @@ def test_compressed_matches_oracle(dtype, lq, lk):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("h,n", [(3, 1), (3, 63), (2, 64), (3, 65), (2, 128), (3, 129), (2, 200), (3, 1041), (16, 4164), (24, 4096)])
+@pytest.mark.parametrize("h,n", [(3, 1), (3, 63), (2, 64), (3, 65), (2, 128), (3, 129), (2, 200), (3, 1041), (16, 4164), (24, 4096), (33, 4000)])
 def test_dense_sweep_of_the_pipelined_kernel_matches_oracle(dtype, h, n):
     """The attention of the compressed branch without a score buffer runs as a dense sweep of the selection kernel:
     with few query blocks two waves share a block and sweep half of the key tiles each (every case here but the
-    last), otherwise one wave sweeps them all (24 heads x 64 blocks).  One to 66 tiles, ragged last tiles, odd and
-    even tile counts, a last workgroup with a single pair."""
+    last two), otherwise one wave sweeps them all (24 heads x 64 blocks) -- unless the waves fill the chip a whole
+    number of times plus a small rest, which again takes two waves per block (33 heads x 63 blocks = 2048 + 31).  One
+    to 66 tiles, ragged last tiles, odd and even tile counts, a last workgroup with a single pair."""
     q = _randn((1, h, n, 64), n, dtype, 0.5)
     k = _randn((1, h, n, 64), n + 1, dtype, 0.5)
     v = _randn((1, h, n, 64), n + 2, dtype)
