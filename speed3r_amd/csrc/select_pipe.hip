@@ -40,6 +40,21 @@
 // compiler then knows that a read of one does not depend on a transfer into another).  A half
 // buffer is refilled (buffer_load ... lds, 16 bytes per lane) right after its fragments have been read,
 // two phases before it is needed again.
+//
+// Shared tiles.  A CU's vector-cache -> LDS path moves 64 bytes per cycle; with private tiles a wave needs 8 KB per
+// 16 MFMAs (512 matrix cycles), the four SIMDs together exactly those 64 bytes per cycle: the transfers, not the matrix
+// pipe, set the pace.  Where the four query blocks of a workgroup walk the same key tiles -- always in a dense sweep,
+// and in the list instance whenever the four lists hold the same blocks (neighbouring query blocks mostly do) -- the
+// workgroup fetches every half tile ONCE: each wave transfers a quarter of it (one instruction of 1 KB) into a ring of
+// four K halves and four V halves shared by the workgroup, and all four waves read their fragments from there.  One
+// workgroup barrier per phase: behind it every wave's quarter of the halves read in this phase has landed and every
+// wave has finished reading the halves of the phase before, which are the ones refilled in this phase (three phases
+// ahead of their use).
+//
+// The queries are multiplied by scale * log2(e) once, in registers, and rounded back to the I/O type: the scores leave
+// the matrix pipe as exponents of two and the loop spends no instruction on scaling them.  bf16 has fp32's exponent
+// range, so its instance uses no softmax reference at all in the loop (exp2 of the score itself; row sums outside
+// [2^-80, 2^100] send the query block to the online-softmax stage); fp16 subtracts the first half tile's row maximum.
 #include "select_common.h"
 #include "attn_params.h"
 
@@ -48,24 +63,36 @@ namespace pipe {
 using namespace sel;
 
 constexpr int kHalf = 32 * 64;  // elements per half tile
-#ifndef S3R_PIPE_WAVES
-#define S3R_PIPE_WAVES 4
-#endif
-constexpr int kWaves = S3R_PIPE_WAVES;  // wavefronts (= query blocks) per workgroup; the waves do not interact
+constexpr int kWaves = 4;  // wavefronts (= query blocks) per workgroup
 
 // DENSE: no index list, every query block attends to all key tiles in order (the compressed branch's attention over
 // the pooled tokens runs through this instance).
 // SPLIT (with DENSE, for sweeps with too few query blocks to fill the chip): two waves share a query block, each
 // sweeps half of the key tiles, and the first one folds the second one's accumulators into its own through LDS.
-template <typename E, bool DENSE, bool SPLIT = false>
+// EXACT (chosen when the caller asks for the log-sum-exp, i.e. for a backward pass that recomputes the probabilities from
+// it): the queries stay as they are in memory and every fp32 score is scaled in the loop, as the reference kernel does.
+template <typename E, bool DENSE, bool SPLIT, bool EXACT>
 __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams p, int nqb, int nqg, int total_wg) {
   static_assert(!SPLIT || DENSE, "the split sweep is a variant of the dense one");
+  constexpr bool ALWAYS_SHARED = DENSE && !SPLIT;            // every query block of a dense sweep walks the same tiles
+  constexpr bool NOREF = std::is_same<E, bf16_t>::value && !EXACT;  // no softmax reference inside the loop
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0[kWaves * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1[kWaves * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0[kWaves * kHalf * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1[kWaves * kHalf * 2];
+  // Separate arrays: the compiler then knows that a read of one does not depend on a transfer into another.
+  // Private tiles: four arrays of 16 KB, a wave's K half 0 / K half 1 / V half 0 / V half 1 buffer is its 4 KB of
+  // k0a / k1a / v0a / v1a.  Shared tiles: eight arrays of 8 KB, ring slot j of K is the first 4 KB of the j-th k array,
+  // ring slot j of V the first 4 KB of the j-th v array; a wave's own 4 KB (staged Q block, unpipelined stage) are
+  // waves 0,1 in the a arrays, waves 2,3 in the b arrays.
+  constexpr int kArrA = ALWAYS_SHARED ? 2 * kHalf * 2 : kWaves * kHalf * 2;
+  constexpr int kArrB = ALWAYS_SHARED ? 2 * kHalf * 2 : 16;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0a[kArrA];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k0b[kArrB];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1a[kArrA];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_k1b[kArrB];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0a[kArrA];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v0b[kArrB];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1a[kArrA];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_v1b[kArrB];
   __shared__ float lds_ml[SPLIT ? kWaves * 4 * 64 : 1];  // SPLIT: per wave and lane the two references and the two row sums
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: addresses derived from it stay scalar
@@ -88,11 +115,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const int h = bh - b * p.H;
   const int split = SPLIT ? (wave & 1) : 0;  // which half of the key tiles
   int qb = SPLIT ? qg * (kWaves / 2) + (wave >> 1) : qg * kWaves + wave;
-  // SPLIT: every wave of the workgroup has to reach the barrier of the hand-over, so a pair past the last query block
-  // repeats the last block's work and stores nothing
-  const bool ghost = SPLIT && qb >= nqb;
-  if (SPLIT) qb = qb < nqb ? qb : nqb - 1;
-  if (qb >= nqb) return;
+  // Every wave of the workgroup has to reach the workgroup's barriers (the hand-over of a split sweep, the phases of
+  // shared tiles, the vote of the list instance), so a wave past the last query block repeats the last block's work
+  // and stores nothing; in the list instance it leaves after the vote.
+  const bool ghost = qb >= nqb;
+  qb = qb < nqb ? qb : nqb - 1;
 
   const int64_t N = p.Lq;
   const int64_t q0 = (int64_t)qb * 64;
@@ -110,13 +137,27 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     __builtin_amdgcn_sched_barrier(0);
   }
 
+  auto region = [&](unsigned char* a, unsigned char* b, int w) -> E* {  // wave w's 4 KB of an array (pair)
+    if constexpr (ALWAYS_SHARED) return reinterpret_cast<E*>((w >> 1) ? b : a) + (w & 1) * kHalf;
+    else return reinterpret_cast<E*>(a) + w * kHalf;
+  };
   auto k_half = [&](auto hf) -> E* {
-    if constexpr (decltype(hf)::value == 0) return reinterpret_cast<E*>(lds_k0) + wave * kHalf;
-    else return reinterpret_cast<E*>(lds_k1) + wave * kHalf;
+    if constexpr (decltype(hf)::value == 0) return region(lds_k0a, lds_k0b, wave);
+    else return region(lds_k1a, lds_k1b, wave);
   };
   auto v_half = [&](auto hf) -> E* {
-    if constexpr (decltype(hf)::value == 0) return reinterpret_cast<E*>(lds_v0) + wave * kHalf;
-    else return reinterpret_cast<E*>(lds_v1) + wave * kHalf;
+    if constexpr (decltype(hf)::value == 0) return region(lds_v0a, lds_v0b, wave);
+    else return region(lds_v1a, lds_v1b, wave);
+  };
+  // the private-tile loop names its buffers through ONE array each (a pointer that may point into either array of a
+  // pair would make the compiler wait for every transfer in flight)
+  auto k_half_of = [&](auto hf, auto) -> E* {
+    static_assert(!ALWAYS_SHARED, "private tiles only");
+    return reinterpret_cast<E*>(decltype(hf)::value == 0 ? lds_k0a : lds_k1a) + wave * kHalf;
+  };
+  auto v_half_of = [&](auto hf, auto) -> E* {
+    static_assert(!ALWAYS_SHARED, "private tiles only");
+    return reinterpret_cast<E*>(decltype(hf)::value == 0 ? lds_v0a : lds_v1a) + wave * kHalf;
   };
   typedef std::integral_constant<int, 0> H0;
   typedef std::integral_constant<int, 1> H1;
@@ -167,7 +208,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     n_ragged = __popcll(__ballot(my_valid && my_idx == ragged_blk));
     n_full = __popcll(todo);
   }
-  if (!SPLIT && n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
+  if (!SPLIT && !ALWAYS_SHARED && ghost) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer may still write LDS when the wave ends
+    return;
+  }
+  if (!SPLIT && !ALWAYS_SHARED && n_full + n_ragged == 0 && p.merge_out == nullptr) {  // nothing to attend to: zeros (the merge path goes on and merges zeros)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer may still write LDS when the wave ends
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
@@ -209,23 +254,47 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   // the instruction's immediate offset moves the LDS side AND the global side by i KB: the scalar offset makes up the rest
   const uint32_t k_step = 8u * (uint32_t)p.skn * (uint32_t)sizeof(E) - 1024u;
   const uint32_t v_step = 8u * (uint32_t)p.svn * (uint32_t)sizeof(E) - 1024u;
-  auto dma_k = [&](auto hf, int64_t start) {  // keys start + 32*hf .. +31
+  auto dma_k = [&](auto hf, auto ab, int64_t start) {  // keys start + 32*hf .. +31
     constexpr int HF = decltype(hf)::value;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + (start + 32 * HF) * p.skn), 0, 0x7fffffff, 0x00020000);
-    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)k_half(hf);
+    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)k_half_of(hf, ab);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[0], 0, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[1], k_step, 1024, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[0], 2 * k_step, 2048, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff[1], 3 * k_step, 3072, 0);
   };
-  auto dma_v = [&](auto hf, int64_t start) {
+  auto dma_v = [&](auto hf, auto ab, int64_t start) {
     constexpr int HF = decltype(hf)::value;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + (start + 32 * HF) * p.svn), 0, 0x7fffffff, 0x00020000);
-    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)v_half(hf);
+    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)v_half_of(hf, ab);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, v_voff, 0, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, v_voff, v_step, 1024, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, v_voff, 2 * v_step, 2048, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, v_voff, 3 * v_step, 3072, 0);
+  };
+  // Shared tiles: ring slots (the V slots overlap the staged Q blocks of waves 0 and 2, so the first V transfers wait
+  // for a barrier behind everybody's read of Q).  A wave moves rows 8*wave .. 8*wave+7 of a half: what instruction
+  // number `wave` of dma_k / dma_v moves.
+  auto k_ring = [&](auto r) -> E* {
+    constexpr int R = decltype(r)::value;
+    return reinterpret_cast<E*>(R == 0 ? lds_k0a : R == 1 ? lds_k0b : R == 2 ? lds_k1a : lds_k1b);
+  };
+  auto v_ring = [&](auto r) -> E* {
+    constexpr int R = decltype(r)::value;
+    return reinterpret_cast<E*>(R == 0 ? lds_v0a : R == 1 ? lds_v0b : R == 2 ? lds_v1a : lds_v1b);
+  };
+  const uint32_t k_voff_w = (wave & 1) ? k_voff[1] : k_voff[0];
+  const uint32_t k_soff_w = (uint32_t)wave * 8u * (uint32_t)p.skn * (uint32_t)sizeof(E);
+  const uint32_t v_soff_w = (uint32_t)wave * 8u * (uint32_t)p.svn * (uint32_t)sizeof(E);
+  auto dma_k_piece = [&](auto r, int64_t first_key) {  // this wave's quarter of keys first_key .. +31 into ring slot r
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(kp + first_key * p.skn), 0, 0x7fffffff, 0x00020000);
+    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)(reinterpret_cast<char*>(k_ring(r)) + wave * 1024);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, k_voff_w, k_soff_w, 0, 0);
+  };
+  auto dma_v_piece = [&](auto r, int64_t first_key) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(vp + first_key * p.svn), 0, 0x7fffffff, 0x00020000);
+    __attribute__((address_space(3))) void* dst = (__attribute__((address_space(3))) void*)(reinterpret_cast<char*>(v_ring(r)) + wave * 1024);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, v_voff, v_soff_w, 0, 0);
   };
   // Every read of a half buffer is preceded by an explicit wait for its transfer (the compiler's own bookkeeping of
   // transfers into LDS is not relied on).  vmcnt counts in issue order; in the loop, and in the start-up sequence,
@@ -237,8 +306,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   auto reads_done = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };  // lgkmcnt(0)
   // ---- LDS -> registers ----
   const int kr_off = c * 128 + ((hh ^ k_swizzle(c)) << 4);
-  auto read_k = [&](auto hf, V8 (&dst)[4]) {  // A operand: lane = key row, head_dim chunk hh + 2*ks
-    const char* kbase = reinterpret_cast<const char*>(k_half(hf));
+  auto read_k_at = [&](const E* buf, V8 (&dst)[4]) {  // A operand: lane = key row, head_dim chunk hh + 2*ks
+    const char* kbase = reinterpret_cast<const char*>(buf);
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
       Frag f;
@@ -250,8 +319,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   const int tr_row = 4 * hh + (i16 >> 2);
   const int tr_chunk = (((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1)) ^ (((tr_row >> 1) & 1) << 2);
   const int tr_off = tr_row * 128 + tr_chunk * 16 + (i16 & 1) * 8;
-  auto read_v = [&](auto hf, V8 (&dst)[2][2]) {  // V^T fragments [jj][dt]: keys 16jj + {4hh.., 8+4hh..} of the half
-    const char* vbase = reinterpret_cast<const char*>(v_half(hf));
+  auto read_v_at = [&](const E* buf, V8 (&dst)[2][2]) {  // V^T fragments [jj][dt]: keys 16jj + {4hh.., 8+4hh..} of the half
+    const char* vbase = reinterpret_cast<const char*>(buf);
 #pragma unroll
     for (int jj = 0; jj < 2; jj++)
 #pragma unroll
@@ -263,23 +332,24 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         dst[jj][dt] = as_v8<E>(f);
       }
   };
+  auto read_v = [&](auto hf, V8 (&dst)[2][2]) { read_v_at(v_half(hf), dst); };
   auto row_max = [&](const f32x16 (&s)[2]) -> float {  // over this lane's 32 keys and its partner's
     float mx = s[0][0];
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
-    return xh_max(mx) * sl2;
+    return xh_max(mx) * (EXACT ? sl2 : 1.f);
   };
   auto half_max = [&](const f32x16& sc) -> float {  // over this lane's 16 keys of a half tile and its partner's
     float mx = sc[0];
 #pragma unroll
     for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
-    return xh_max(mx) * sl2;
+    return xh_max(mx) * (EXACT ? sl2 : 1.f);
   };
-  auto scores_half = [&](auto hf) {  // st[.][hf] from the K half in LDS
-    constexpr int HF = decltype(hf)::value;
-    read_k(hf, ak);
+  auto scores_half_at = [&](const E* buf) {  // st[.][0] from a K half in LDS
+    constexpr int HF = 0;
+    read_k_at(buf, ak);
 #pragma unroll
     for (int qt = 0; qt < 2; qt++) {
 #pragma unroll
@@ -302,32 +372,53 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
   //   MFMA slots 0..7 : PV of unit u-1 (probabilities pf[.][KT^1], fragments already in vfr)
   //   MFMA slots 8..15: S^T of unit u+1 into st[.][KT^1] (K half KT^1 read at slot 0)
   //   VALU, all slots : exponentials of unit u, st[.][KT] -> pf[.][KT], two elements per slot
-  // After its fragments are read, K half KT^1 is refilled from tile k_next and V half KT from tile v_next.
+  // Private tiles (ring_tag < 0): after its fragments are read, K half KT^1 is refilled from tile k_next and V half KT
+  // from tile v_next.
+  // Shared tiles (ring_tag = unit number mod 4): K half of unit u+1 from ring slot (u+1)%4, V half of unit u from slot
+  // u%4; this wave's quarter of the K half of unit u+4 (first key k_next) goes into slot u%4 and of the V half of unit
+  // u+3 (first key v_next) into slot (u+3)%4, both read in the phase before.  The wait in front of the barrier covers
+  // this wave's quarters of the two halves read here: transfers complete in order, two per phase, and the four issued
+  // since (units u+2, u+3 of K and u+1, u+2 of V) may stay in flight.
   // Empty volatile asm statements on the score tuple before and on the probability tuple after pin the VALU
   // instructions of a slot; the scheduling barrier after every slot keeps the MFMAs where they are written.
   float mneg[2];
-  auto phase = [&](auto kt_tag, int64_t k_next, int64_t v_next) {
+  float px[2] = {0.f, 0.f};  // the exponentials of the slot before
+  auto phase = [&](auto kt_tag, auto ring_tag, int64_t k_next, int64_t v_next) {
     constexpr int KT = decltype(kt_tag)::value;
     constexpr int OT = KT ^ 1;
+    constexpr int U = decltype(ring_tag)::value;
+    constexpr bool SH = U >= 0;
     typedef std::integral_constant<int, OT> HO;
+    typedef std::integral_constant<int, SH ? 0 : -1 - U> AB;  // private tiles: ring_tag -1 = a arrays, -2 = b arrays
     static_for<16>([&](auto j_tag) {
       constexpr int j = decltype(j_tag)::value;
-      // a half buffer is refilled two slots after its fragments were requested, once they have arrived
-      if constexpr (j == 0) {
-        wait_transfer();
-        read_k(HO{}, ak);
-      }
-      if constexpr (j == 2) {
-        reads_done();
-        dma_k(HO{}, k_next);
-      }
-      if constexpr (j == 8) {
-        wait_transfer();
-        read_v(kt_tag, vfr);
-      }
-      if constexpr (j == 10) {
-        reads_done();
-        dma_v(kt_tag, v_next);
+      if constexpr (SH) {
+        if constexpr (j == 0) {
+          __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4), lgkmcnt(0)
+          __builtin_amdgcn_s_barrier();
+          read_k_at(k_ring(std::integral_constant<int, (U + 1) & 3>{}), ak);
+        }
+        if constexpr (j == 2) dma_k_piece(std::integral_constant<int, U & 3>{}, k_next);
+        if constexpr (j == 8) read_v_at(v_ring(std::integral_constant<int, U & 3>{}), vfr);
+        if constexpr (j == 10) dma_v_piece(std::integral_constant<int, (U + 3) & 3>{}, v_next);
+      } else {
+        // a half buffer is refilled two slots after its fragments were requested, once they have arrived
+        if constexpr (j == 0) {
+          wait_transfer();
+          read_k_at(k_half_of(HO{}, AB{}), ak);
+        }
+        if constexpr (j == 2) {
+          reads_done();
+          dma_k(HO{}, AB{}, k_next);
+        }
+        if constexpr (j == 8) {
+          wait_transfer();
+          read_v_at(v_half_of(kt_tag, AB{}), vfr);
+        }
+        if constexpr (j == 10) {
+          reads_done();
+          dma_v(kt_tag, AB{}, v_next);
+        }
       }
       if constexpr (j < 8) {
         constexpr int jj = j >> 2, dt = (j >> 1) & 1, qt = j & 1;
@@ -344,26 +435,34 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         }
       }
       {
+        // The slot starts the two exponentials of its own pair of scores and rounds and sums the pair of the slot
+        // BEFORE it (the first slot: the last pair of the unit before, whose probabilities the PV stage needs from
+        // its sixth slot on): nothing in a slot waits for an exponential started in the same slot.
         constexpr int e = 2 * j;
-        constexpr int qt = e >> 4, r = e & 15, jj = r >> 3, e8 = r & 7;
+        constexpr int qt = e >> 4, r = e & 15;
+        constexpr int pe = (e + 30) & 31, PT = j == 0 ? OT : KT;
+        constexpr int pqt = pe >> 4, pjj = (pe & 15) >> 3, pe8 = pe & 7;
         asm volatile("" : "+v"(st[qt][KT]));
-        const float x0 = __builtin_amdgcn_exp2f(fmaf(st[qt][KT][r], sl2, mneg[qt]));
-        const float x1 = __builtin_amdgcn_exp2f(fmaf(st[qt][KT][r + 1], sl2, mneg[qt]));
+        const float x0 = __builtin_amdgcn_exp2f(EXACT ? fmaf(st[qt][KT][r], sl2, mneg[qt]) : NOREF ? st[qt][KT][r] : st[qt][KT][r] + mneg[qt]);
+        const float x1 = __builtin_amdgcn_exp2f(EXACT ? fmaf(st[qt][KT][r + 1], sl2, mneg[qt]) : NOREF ? st[qt][KT][r + 1] : st[qt][KT][r + 1] + mneg[qt]);
         V2 pk;
-        pk[0] = (E)x0;
-        pk[1] = (E)x1;
-        pf[qt][KT][jj][e8] = pk[0];
-        pf[qt][KT][jj][e8 + 1] = pk[1];
+        pk[0] = (E)px[0];
+        pk[1] = (E)px[1];
+        pf[pqt][PT][pjj][pe8] = pk[0];
+        pf[pqt][PT][pjj][pe8 + 1] = pk[1];
         // row sums over the unrounded probabilities, as the reference's tl.sum(p) before p.to(v.dtype); the pair is
-        // added first: two additions chained on the sum stall the second one behind the exponential's result
-        l_i[qt] += x0 + x1;
-        asm volatile("" : "+v"(pf[qt][KT][jj]), "+v"(l_i[qt]));
+        // added first: two additions chained on the sum stall the second one
+        l_i[pqt] += px[0] + px[1];
+        px[0] = x0;
+        px[1] = x1;
+        asm volatile("" : "+v"(pf[pqt][PT][pjj]), "+v"(l_i[pqt]), "+v"(px[0]), "+v"(px[1]));
       }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
 
   // Unpipelined stage with a true online softmax: one key tile (possibly ragged) from global memory.
+  float qs = EXACT ? sl2 : 1.f;  // what a score of the unpipelined stage is still to be multiplied by: 1 while the queries carry the scale
   auto robust_tile = [&](int64_t start) {
     const int nvalid = (int)((N - start < 64) ? (N - start) : 64);
     const E* kb = kp + start * p.skn;
@@ -403,7 +502,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
 #pragma unroll
         for (int r = 0; r < 16; r++)
           if (kt * 32 + 8 * (r >> 2) + (r & 3) >= lim) st[qt][kt][r] = -INFINITY;
-      const float mx = row_max(st[qt]);
+      const float mx = row_max(st[qt]) * (EXACT ? 1.f : qs);
       const float m_new = fmaxf(m_i[qt], mx);
       const float alpha = __builtin_amdgcn_exp2f(m_i[qt] - m_new);  // 0 on the first tile (m_i = -inf)
       m_i[qt] = m_new;
@@ -418,8 +517,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         for (int jj = 0; jj < 2; jj++)
 #pragma unroll
           for (int e = 0; e < 8; e += 2) {
-            const float x0 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e], sl2, -m_new));
-            const float x1 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e + 1], sl2, -m_new));
+            const float x0 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e], qs, -m_new));
+            const float x1 = __builtin_amdgcn_exp2f(fmaf(st[qt][kt][8 * jj + e + 1], qs, -m_new));
             pf[qt][kt][jj][e] = (E)x0;
             pf[qt][kt][jj][e + 1] = (E)x1;
             l_i[qt] += x0 + x1;
@@ -439,15 +538,29 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
         for (int r = 0; r < 16; r++) ot[dt][qt][r] = 0.f;
     m_i[0] = m_i[1] = -INFINITY;
     l_i[0] = l_i[1] = 0.f;
+    // ... and the queries as they are in memory: the recomputation scales the fp32 scores, like the reference kernel
+    if constexpr (EXACT) return;
+    const int q_last = (int)((N - q0 < 64 ? N - q0 : 64) - 1);
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+      const int row = 32 * qt + c < q_last ? 32 * qt + c : q_last;
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(qp + (q0 + row) * p.sqm + (hh + 2 * ks) * 8);
+        bq[qt][ks] = as_v8<E>(f);
+      }
+    }
+    qs = sl2;
   };
 
   bool redo = false;
   // Operands of the gated merge (epilogue): gate pair per query row, the query block's row of the compressed output
-  // in this lane's store layout.  Issued right after the main loop, so that their latency passes behind the last PV
+  // in the layout of this lane's accumulators.  Issued right after the main loop, so that their latency passes behind the last PV
   // stage instead of in front of the stores.
   const bool merge = p.merge_out != nullptr;
   uint32_t g_raw[2] = {0, 0};  // gate pair per query row, bits of the I/O type
-  uint4 oc_raw[2][2];  // [dt][gp]
+  uint2 oc_raw[2][4];  // [dt][g4]: this lane's four head_dim values of group g4, the accumulators' own layout
   bool merge_loaded = false;
   auto load_merge_operands = [&]() {
     if (merge) {
@@ -463,7 +576,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
 #pragma unroll
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-        for (int gp = 0; gp < 2; gp++) oc_raw[dt][gp] = *reinterpret_cast<const uint4*>(ocp + dt * 32 + 8 * (2 * gp + hh));
+        for (int g4 = 0; g4 < 4; g4++) oc_raw[dt][g4] = *reinterpret_cast<const uint2*>(ocp + dt * 32 + 8 * g4 + 4 * hh);
     }
     merge_loaded = true;
   };
@@ -480,6 +593,14 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
       }
     }
     reads_done();  // before the V buffers are refilled
+    // the queries carry the softmax scale and the change of base from here on (one rounding to the I/O type)
+    if constexpr (!EXACT)
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) bq[qt][ks][e] = (E)((float)bq[qt][ks][e] * sl2);
   };
   if (n_full == 0) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the Q transfers have landed
@@ -500,48 +621,122 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
       last_start = any ? s : last_start;
       return last_start;
     };
-    const int64_t s0 = pop_or_last();
-    // transfers in the rotation of the loop (K1, V0, K0, V1), so that the loop's waits hold from the first phase on
-    dma_k(H0{}, s0);
-    dma_k(H1{}, s0);
-    __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the Q transfers, issued before these eight, have landed
-    read_q();
-    dma_v(H0{}, s0);
-    int64_t s1 = pop_or_last(), s2 = pop_or_last();
-    // the row maxima over the first half tile become the softmax reference; st[.][0] stays for the first phase
-    __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the first K half
-    scores_half(H0{});
-    reads_done();
-    dma_k(H0{}, s1);  // the K half the second phase reads
-
-    dma_v(H1{}, s0);
-    m_i[0] = half_max(st[0][0]);
-    m_i[1] = half_max(st[1][0]);
-    mneg[0] = -m_i[0];
-    mneg[1] = -m_i[1];
+    // the first half tile's scores are in st[.][0]: softmax reference (fp16 only: its row maxima), nothing for the first
+    // phase's PV stage to add
+    auto first_unit_done = [&]() {
+      if constexpr (NOREF) {
+        m_i[0] = m_i[1] = 0.f;
+      } else {
+        m_i[0] = half_max(st[0][0]);
+        m_i[1] = half_max(st[1][0]);
+      }
+      mneg[0] = -m_i[0];
+      mneg[1] = -m_i[1];
 #pragma unroll
-    for (int qt = 0; qt < 2; qt++)  // the first phase's PV stage adds nothing
+      for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) pf[qt][1][jj][e] = (E)0.f;
 #pragma unroll
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) pf[qt][1][jj][e] = (E)0.f;
+        for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-    for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-      for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) vfr[jj][dt][e] = (E)0.f;
-    for (int i = n_full; i > 0; i--) {  // past the end of the list the transfers re-read the last tile
-      phase(H0{}, s1, s1);
-      phase(H1{}, s2, s1);
-      s1 = s2;
-      s2 = pop_or_last();
+          for (int e = 0; e < 8; e++) vfr[jj][dt][e] = (E)0.f;
+    };
+    typedef std::integral_constant<int, 0> U0;
+    typedef std::integral_constant<int, 1> U1;
+    typedef std::integral_constant<int, 2> U2;
+    typedef std::integral_constant<int, 3> U3;
+    if constexpr (ALWAYS_SHARED) {
+      // Units 0..3 of K and 0..2 of V, in the order the loop goes on with (K of unit u+4, V of unit u+3 in phase u).
+      int64_t sa = pop_or_last(), sb = pop_or_last();
+      dma_k_piece(U0{}, sa);
+      dma_k_piece(U1{}, sa + 32);
+      dma_k_piece(U2{}, sb);
+      dma_k_piece(U3{}, sb + 32);
+      __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4): the Q transfers, issued before these four, have landed
+      read_q();                            // (ends with lgkmcnt(0))
+      __builtin_amdgcn_s_barrier();        // every wave has read its Q block: the V slots are free
+      dma_v_piece(U0{}, sa);
+      dma_v_piece(U1{}, sa + 32);
+      dma_v_piece(U2{}, sb);
+      __builtin_amdgcn_s_waitcnt(0x0F76);  // vmcnt(6): this wave's quarter of the first K half ...
+      __builtin_amdgcn_s_barrier();        // ... and the other three
+      scores_half_at(k_ring(U0{}));
+      first_unit_done();
+      // The loop's wait (four transfers may stay in flight) assumes its own issue order, K of unit u+4 and V of unit
+      // u+3 in phase u; the start-up sent K ahead of V, so everything sent so far has to land before the first phase.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      for (int i = n_full >> 1; i > 0; i--) {  // two tiles per round; past the end of the list the transfers re-read the last tile
+        const int64_t sc = pop_or_last(), sd = pop_or_last();
+        phase(H0{}, U0{}, sc, sb + 32);
+        phase(H1{}, U1{}, sc + 32, sc);
+        phase(H0{}, U2{}, sd, sc + 32);
+        phase(H1{}, U3{}, sd + 32, sd);
+        sb = sd;
+      }
+      if (n_full & 1) {  // the ring is back at slot 0 after every round
+        const int64_t sc = pop_or_last();
+        phase(H0{}, U0{}, sc, sb + 32);
+        phase(H1{}, U1{}, sc + 32, sc);
+      }
+    } else {
+      auto run_private = [&](auto ab) {  // ab = 0: this wave's buffers are in the a arrays, 1: in the b arrays
+        typedef std::integral_constant<int, -1 - decltype(ab)::value> Priv;
+        const int64_t s0 = pop_or_last();
+        // transfers in the rotation of the loop (K1, V0, K0, V1), so that the loop's waits hold from the first phase on
+        dma_k(H0{}, ab, s0);
+        dma_k(H1{}, ab, s0);
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the Q transfers, issued before these eight, have landed
+        read_q();
+        dma_v(H0{}, ab, s0);
+        int64_t s1 = pop_or_last(), s2 = pop_or_last();
+        __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): the first K half
+        scores_half_at(k_half_of(H0{}, ab));
+        reads_done();
+        dma_k(H0{}, ab, s1);  // the K half the second phase reads
+
+        dma_v(H1{}, ab, s0);
+        first_unit_done();
+        for (int i = n_full; i > 0; i--) {  // past the end of the list the transfers re-read the last tile
+          phase(H0{}, Priv{}, s1, s1);
+          phase(H1{}, Priv{}, s2, s1);
+          s1 = s2;
+          s2 = pop_or_last();
+        }
+      };
+      run_private(std::integral_constant<int, 0>{});
+    }
+    if constexpr (ALWAYS_SHARED) {
+      // the later stages write the V slots' memory (every wave its own 4 KB): nobody may still read a slot, and no
+      // transfer (the last ones re-read the last tile) may still be on its way into one
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
     }
     load_merge_operands();
+    {  // the last pair of the last unit
+      V2 pk;
+      pk[0] = (E)px[0];
+      pk[1] = (E)px[1];
+      pf[1][1][1][6] = pk[0];
+      pf[1][1][1][7] = pk[1];
+      l_i[1] += px[0] + px[1];
+    }
     pv_half(H1{});  // PV of the last unit
-    // a reference that was too low shows up as a huge or non-finite row sum
-    const float big = 1.2676506e30f;  // 2^100
+    // The row sums tell whether the loop's shortcuts held.  They add the unrounded fp32 probabilities, all of them
+    // >= 0, so a lane's sum is at least as large as each of its probabilities.
+    //  * fp16: a sum below 65504 proves that no probability left fp16's range when it was rounded (the reference, the
+    //    first half tile's row maximum, may lie below later scores).
+    //  * bf16 (no reference, exp2 of the score itself): a sum below 2^20 proves that every score (times scale*log2(e))
+    //    was below 20, a row total above 2^-20 that its largest one was above -20.  Inside that band the rounding of
+    //    the scaled queries to bf16 (2^-9 of each product) moves a score by about a thousandth of the band's width or
+    //    less; outside it the query block is recomputed from the queries as they are in memory.
+    //  * EXACT, bf16: the reference is the first half tile's row maximum, a later score may exceed it by 100.
+    const float big = NOREF ? 1048576.f : std::is_same<E, f16_t>::value ? 65504.f : 1.2676506e30f;
     redo = __any(!(l_i[0] < big) || !(l_i[1] < big));
+    if constexpr (NOREF) redo = redo || __any(!(xh_sum(l_i[0]) > 9.5367e-7f) || !(xh_sum(l_i[1]) > 9.5367e-7f));
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no transfer is still writing LDS
 
@@ -567,8 +762,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     // the second wave of a pair hands its state over: accumulators [dt][qt] into its four (now idle) 4 KB buffers,
     // register r of lane l at float r*64 + l, references and row sums into lds_ml; the first wave folds them in
     auto xo = [&](int w, int dt, int qt) -> float* {
-      unsigned char* a = dt == 0 ? (qt == 0 ? lds_k0 : lds_k1) : (qt == 0 ? lds_v0 : lds_v1);
-      return reinterpret_cast<float*>(a + w * (kHalf * 2));
+      return reinterpret_cast<float*>(dt == 0 ? (qt == 0 ? region(lds_k0a, lds_k0b, w) : region(lds_k1a, lds_k1b, w))
+                                              : (qt == 0 ? region(lds_v0a, lds_v0b, w) : region(lds_v1a, lds_v1b, w)));
     };
     if (split == 1) {
 #pragma unroll
@@ -611,13 +806,29 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
     g0[qt] = (float)lo.e;
     g1[qt] = (float)hi.e;
   }
+  // With the merge the stored value is gate0 * o_cmp + gate1 * (accumulator / row sum), evaluated in fp32 and rounded
+  // ONCE: the selection output is never rounded on its own, nor are the two products (the eager expression rounds all
+  // three and the sum: at most two rounding steps of the I/O type away, on the side of the exact value).
+  float ocf[2][16];
+  if (merge) {
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const V2 lo2 = __builtin_bit_cast(V2, oc_raw[dt][g4].x), hi2 = __builtin_bit_cast(V2, oc_raw[dt][g4].y);
+        ocf[dt][4 * g4] = (float)lo2[0];
+        ocf[dt][4 * g4 + 1] = (float)lo2[1];
+        ocf[dt][4 * g4 + 2] = (float)hi2[0];
+        ocf[dt][4 * g4 + 3] = (float)hi2[1];
+      }
+  }
 #pragma unroll
   for (int qt = 0; qt < 2; qt++) {
-#pragma clang fp contract(off)  // the merge rounds each product and the sum separately, like the eager expression
     const float l = xh_sum(l_i[qt]);
     const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float ginv = g1[qt] * inv;
     const int64_t row = q0 + qt * 32 + c;
-    const bool live = row < N;
+    const bool live = row < N && !(ALWAYS_SHARED && ghost);
 #pragma unroll
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -630,32 +841,22 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_pipe_kernel(AttnParams 
           v[1] = (E)y;
           return __builtin_bit_cast(uint32_t, v);
         };
+        auto value = [&](int r) -> float {
+          return merge ? fmaf(ot[dt][qt][r], ginv, g0[qt] * ocf[dt][r]) : ot[dt][qt][r] * inv;
+        };
         union { uint32_t w[4]; uint4 u; } pc;
 #pragma unroll
         for (int wi = 0; wi < 2; wi++) {
-          const uint32_t a = pack2(ot[dt][qt][8 * gp + 2 * wi] * inv, ot[dt][qt][8 * gp + 2 * wi + 1] * inv);
-          const uint32_t bw = pack2(ot[dt][qt][8 * gp + 4 + 2 * wi] * inv, ot[dt][qt][8 * gp + 4 + 2 * wi + 1] * inv);
+          const uint32_t a = pack2(value(8 * gp + 2 * wi), value(8 * gp + 2 * wi + 1));
+          const uint32_t bw = pack2(value(8 * gp + 4 + 2 * wi), value(8 * gp + 4 + 2 * wi + 1));
           const auto r = __builtin_amdgcn_permlane32_swap(a, bw, false, false);
           pc.w[wi] = r[0];
           pc.w[2 + wi] = r[1];
         }
         const int d0 = dt * 32 + 8 * (2 * gp + hh);
         if (live) {
-          if (!merge) {
-            *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
-          } else {
-            union { uint32_t w[4]; uint4 u; } oc, res;
-            oc.u = oc_raw[dt][gp];
-#pragma unroll
-            for (int wi = 0; wi < 4; wi++) {  // products and sum each rounded to the I/O type, as the eager expression does
-              const V2 o2 = __builtin_bit_cast(V2, oc.w[wi]);
-              const V2 s2 = __builtin_bit_cast(V2, pc.w[wi]);
-              const V2 x2 = __builtin_bit_cast(V2, pack2(g0[qt] * (float)o2[0], g0[qt] * (float)o2[1]));
-              const V2 y2 = __builtin_bit_cast(V2, pack2(g1[qt] * (float)s2[0], g1[qt] * (float)s2[1]));
-              res.w[wi] = pack2((float)x2[0] + (float)y2[0], (float)x2[1] + (float)y2[1]);
-            }
-            *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = res.u;
-          }
+          if (!merge) *reinterpret_cast<uint4*>(op + row * p.som + d0) = pc.u;
+          else *reinterpret_cast<uint4*>((E*)p.merge_out + (((int64_t)b * N + row) * p.H + h) * 64 + d0) = pc.u;
         }
       }
     if (live && p.lse != nullptr && hh == 0)
@@ -681,14 +882,20 @@ int launch_select_pipe(const AttnParams& p, int dtype, void* stream) {
   if (total > 0x7fffffffLL) return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn: grid too large");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)total), blk(64 * pipe::kWaves);
-#define S3R_PIPE_LAUNCH(E)                                                                                                       \
+#define S3R_PIPE_LAUNCH(E, X)                                                                                                      \
   do {                                                                                                                           \
-    if (split) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total); \
-    else if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);  \
-    else hipLaunchKernelGGL((pipe::select_pipe_kernel<E, false>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);            \
+    if (split) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true, true, X>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);       \
+    else if (dense) hipLaunchKernelGGL((pipe::select_pipe_kernel<E, true, false, X>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total); \
+    else hipLaunchKernelGGL((pipe::select_pipe_kernel<E, false, false, X>), grid, blk, 0, st, p, (int)nqb, (int)nqg, (int)total);           \
   } while (0)
-  if (dtype == S3R_BF16) S3R_PIPE_LAUNCH(bf16_t);
-  else S3R_PIPE_LAUNCH(f16_t);
+  const bool exact = p.lse != nullptr;  // a caller that wants the log-sum-exp wants it to the reference's precision
+  if (dtype == S3R_BF16) {
+    if (exact) S3R_PIPE_LAUNCH(bf16_t, true);
+    else S3R_PIPE_LAUNCH(bf16_t, false);
+  } else {
+    if (exact) S3R_PIPE_LAUNCH(f16_t, true);
+    else S3R_PIPE_LAUNCH(f16_t, false);
+  }
 #undef S3R_PIPE_LAUNCH
   return check_launch("select_pipe_kernel");
 }

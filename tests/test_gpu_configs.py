@@ -1,8 +1,8 @@
 """Whole-path parity at the benchmark configurations (needs an MI355X).
 
-config 1 (fp32, 8 frames) is checked against the CPU oracle in full; config 2 (bf16, 64 frames)
-on a slice of heads the oracle finishes in seconds; config 3 (bf16, 256 frames, the headline
-shape) through size-independent properties plus an oracle comparison on sampled rows.
+config 1 (fp32, 8 frames), config 2 (bf16, 64 frames) and config 3 (bf16, 256 frames, the headline
+shape) are checked against the CPU oracle in full, all 16 heads; config 3 also through
+size-independent properties, config 4 (1000 frames) through properties and sampled query blocks.
 """
 import numpy as np
 import pytest
@@ -12,7 +12,7 @@ import torch.nn.functional as F
 import oracle
 import speed3r_amd as s3r
 from speed3r_amd import workloads
-from helpers import max_abs
+from helpers import max_abs, merged_within_rounding
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -44,25 +44,48 @@ def test_config1_fp32_full_path_vs_oracle():
         assert max_abs(out, oracle.gated_merge(ref["o_cmp"], o_sel_ref, gate, 64)) <= 1e-5
 
 
-def test_config2_bf16_vs_fp32_oracle_on_head_slice():
-    cfg, q, k, v, gate = workloads.make_config("cfg2")
+def _whole_path_against_the_oracle(cfg, q, k, v, gate):
+    """Every head of a bf16 configuration against the oracle on the same (already rounded) inputs: pooled tensors,
+    compressed attention, index overlap (near-ties may go the other way between bf16 and fp32 statistics), selection
+    on the ORACLE's indices, the device's selection on the DEVICE's indices, and the merged output."""
     qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, gate))
+    n, h = cfg.tokens, q.shape[1]
     out, parts = s3r.sparse_global_attention(qd, kd, vd, gd, 64, cfg.topk, return_parts=True)
-    assert out.shape == (1, cfg.tokens, 1024)
-    hs = slice(0, 2)
-    ref = oracle.sparse_global_attention(q[:, hs], k[:, hs], v[:, hs], gate[:, hs], 64, cfg.topk)
-    assert max_abs(parts["qc"][:, hs], ref["qc"]) <= 2e-2
-    assert max_abs(parts["o_cmp"][:, hs], ref["o_cmp"]) <= 2e-2
-    ov = _overlap(parts["idx"][:, hs], ref["idx"])
-    assert ov >= 0.97, f"index overlap with the fp32 oracle {ov}"      # near-ties may flip between bf16 and fp32
-    # selection given the oracle's indices, and merge given the oracle's parts
-    o_sel = s3r.select_attn(qd[:, hs], kd[:, hs], vd[:, hs], ref["idx"].to(DEV), 64)
+    assert out.shape == (1, n, h * 64)
+    ref = oracle.sparse_global_attention(q, k, v, gate, 64, cfg.topk)
+    assert max_abs(parts["qc"], ref["qc"]) <= 2e-2
+    assert max_abs(parts["o_cmp"], ref["o_cmp"]) <= 2e-2
+    ov = _overlap(parts["idx"], ref["idx"])
+    assert ov >= 0.97, f"index overlap with the fp32 oracle {ov}"
+    o_sel = s3r.select_attn(qd, kd, vd, ref["idx"].to(DEV), 64)
     assert max_abs(o_sel, ref["o_sel"].float()) <= 2e-2
-    o_sel_ref = oracle.select_attention(q[:, hs], k[:, hs], v[:, hs], parts["idx"][:, hs].cpu(), 64, out_dtype=torch.float32)
-    assert max_abs(parts["o_sel"][:, hs], o_sel_ref) <= 2e-2
-    want = oracle.gated_merge(ref["o_cmp"].float(), o_sel_ref, gate[:, hs].float(), 64)
-    got = out.view(1, cfg.tokens, 16, 64)[:, :, hs].reshape(1, cfg.tokens, 128)
-    assert max_abs(got, want) <= 2e-2
+    del o_sel
+    o_sel_ref = oracle.select_attention(q, k, v, parts["idx"].cpu(), 64, out_dtype=torch.float32)
+    assert max_abs(parts["o_sel"], o_sel_ref) <= 2e-2
+    # Merged output.  Same rounding points as the eager bf16 expression: bit for bit on the device's own parts; against
+    # the merge evaluated in fp32 the bar is 2e-2 absolute up to magnitude 1 and 2e-2 relative above it (the eager
+    # expression rounds both products and the sum to bf16, whose step is 2^-8 of the value: at the headline shape the
+    # low-rank component of v takes outputs to magnitude 3, where ONE rounding step is already 1.6e-2).
+    assert torch.equal(out.cpu(), oracle.gated_merge(parts["o_cmp"].cpu(), parts["o_sel"].cpu(), gate, 64))
+    want = oracle.gated_merge(ref["o_cmp"].float(), o_sel_ref, gate.float(), 64)
+    fused = s3r.sparse_global_attention(qd, kd, vd, gd, 64, cfg.topk)   # merge in the selection kernel's epilogue (layer, benchmark)
+    for got in (out, fused):
+        err = (got.float().cpu() - want).abs()
+        assert (err <= 2e-2 * want.abs().clamp(min=1.0)).all(), f"max abs {err.max().item()}, largest |want| {want.abs().max().item()}"
+    return ov
+
+
+def test_config2_bf16_all_heads_vs_fp32_oracle():
+    cfg, q, k, v, gate = workloads.make_config("cfg2")
+    _whole_path_against_the_oracle(cfg, q, k, v, gate)
+
+
+def test_config3_bf16_all_heads_vs_fp32_oracle():
+    """The headline shape in full: 266 496 tokens, all 16 heads (the oracle takes about ten seconds per pass on the
+    box's 16 host threads)."""
+    cfg, q, k, v, gate = workloads.make_config("cfg3")
+    _whole_path_against_the_oracle(cfg, q, k, v, gate)
+    torch.cuda.empty_cache()
 
 
 @pytest.fixture(scope="module")
@@ -178,8 +201,8 @@ def test_config4_1000_frames_fit_one_gpu_and_hold_their_properties(cfg4_inputs, 
     assert int(idx.min()) >= 0 and int(idx.max()) < nc
     srt = idx.sort(dim=-1).values
     assert (srt[..., 1:] != srt[..., :-1]).all()
-    # the fused path gives the same bits as the two operators
-    assert torch.equal(s3r.sparse_global_attention(q, k, v, gate, 64, topk), out)
+    # the merge in the selection kernel's epilogue (one rounding) against the two operators' parts
+    assert merged_within_rounding(s3r.sparse_global_attention(q, k, v, gate, 64, topk), parts["o_cmp"], parts["o_sel"], gate, 64)
     # pooled ragged tail: mean over the 40 valid tokens
     tail = q[0, :, (nc - 1) * 64:].float().mean(dim=1)
     assert max_abs(parts["qc"][0, :, nc - 1], tail) <= 2e-2
