@@ -7,8 +7,15 @@ workload is the headline configuration: 256 frames x 1041 tokens = 266 496 token
 block 64, top-k 16, bf16, seeded low-rank-plus-noise q/k/v.
 
 Prints ONE JSON line: ms/layer as `value`, effective TFLOP/s, per-kernel times measured with HIP
-events on the launch stream, the roofline of the dominant (selection) kernel from its algorithmic
-FLOPs, and a CPU baseline (the Python oracle timed on this host's cores on a bounded sample).
+events on the launch stream (mean and median), the roofline of the dominant (selection) kernel from
+its algorithmic FLOPs, and a CPU baseline (the Python oracle timed on this host's cores on a bounded
+sample).  The default run appends, each from a short timed loop of its own after the headline region:
+GB/s of the HBM-bound kernels on one stream (`hbm_gbs`), the 1000-frame layer (`cfg4`) and the
+end-to-end model (`cfg5`: frames/s and the share of time inside the sparse attention modules).
+
+The chip's clock governor needs some tens of back-to-back launches to settle under this load (the
+first launches after an idle period run up to 40 % slower), so every timed loop is preceded by a
+fixed number of untimed settling steps (`settle_steps` in the JSON) on top of `--warmup`.
 """
 from __future__ import annotations
 
@@ -25,6 +32,7 @@ if str(ROOT) not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+SETTLE_STEPS = 40           # untimed steps in front of --warmup (clock governor), fixed
 # (config, top-k, block, merge fused) -> HBM bytes per launch of the selection kernel and the profile summary they come from
 MEASURED_TRAFFIC = {
     ("cfg3", 16, 64, True): (2.34e9, "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md"),
@@ -35,10 +43,10 @@ MEASURED_TRAFFIC = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # The chip's clock governor needs some tens of back-to-back launches to settle under this load (the first
-    # launches after an idle period run up to 40 % slower), so the default warm-up is long; a step is 1.8 ms.
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true",
+                    help="headline region only: no hbm_gbs / cfg4 / cfg5 loops after it (profiling runs)")
     ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
                     help="cfg1-cfg4: one sparse global-attention layer call; cfg5: end-to-end Pi3_Sparse-style forward (frames/s)")
     ap.add_argument("--frames", type=int, default=100, help="cfg5: number of 518x392 frames")
@@ -117,7 +125,7 @@ def _prepass_stage(qd, kd, vd, block):
     return lambda: ops.qkv_prepass(packed, h, block, pos, cos, sin, ln[0], ln[1], 1e-6)
 
 
-def run_end_to_end(args) -> int:
+def run_end_to_end(args, steps=None, warmup=None) -> dict:
     """cfg5: random-init Pi3_Sparse-style model, bf16, synthetic frames in [0,1]; frames/s and the share of GPU time
     spent in the sparse global attention (HIP events around the 18 global attention modules)."""
     import torch
@@ -144,9 +152,11 @@ def run_end_to_end(args) -> int:
     for blk in model.global_decoder:
         blk.attn.register_forward_pre_hook(pre)
         blk.attn.register_forward_hook(post)
-    steps, warmup = min(args.steps, 5), min(args.warmup, 2)
+    steps = steps if steps is not None else min(args.steps, 5)
+    warmup = warmup if warmup is not None else max(min(args.warmup, 2), 1)
+    torch.cuda.reset_peak_memory_stats()
     with torch.no_grad():
-        for _ in range(max(warmup, 1)):
+        for _ in range(warmup):
             model(imgs)
         torch.cuda.synchronize()
         spans.clear()
@@ -158,9 +168,9 @@ def run_end_to_end(args) -> int:
     sparse_ms = sum(a.elapsed_time(b) for a, b in spans) / steps
     ms = wall * 1e3 / steps
     tokens = args.frames * 1041
-    print(json.dumps({
+    res = {
         "metric": "frames/s, Pi3_Sparse-style forward (ViT-L/14 encoder + 36-layer decoder + heads), bf16",
-        "value": args.frames / (ms * 1e-3), "unit": "frames/s", "n_gpus": 1, "steps": steps, "warmup": max(warmup, 1),
+        "value": args.frames / (ms * 1e-3), "unit": "frames/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"cfg5: {args.frames} frames 518x392 -> {tokens} tokens (5 register + 1036 patch per frame), "
@@ -170,8 +180,139 @@ def run_end_to_end(args) -> int:
         "sparse_attention_ms_per_layer": sparse_ms / len(model.global_decoder),
         "peak_mem_gb": torch.cuda.max_memory_allocated() / 1e9,
         "outputs": {k: list(v.shape) for k, v in out.items()},
-    }))
-    return 0
+    }
+    del model, imgs, out
+    torch.cuda.empty_cache()
+    return res
+
+
+def time_layer(step, steps, warmup, overlap, fused):
+    """SETTLE_STEPS + `warmup` untimed steps, then exactly `steps` timed ones between two device synchronisations;
+    per-kernel spans from HIP events recorded on the launch stream inside every timed step (mean and median)."""
+    import statistics
+
+    import torch
+
+    with torch.no_grad():
+        for _ in range(SETTLE_STEPS + warmup):
+            step()
+        torch.cuda.synchronize()
+        evs = [{} for _ in range(steps)]
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(evs[i])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    fused = fused and "merge" not in evs[0]   # the merge runs in the selection kernel's epilogue only where that is built
+    spans = {}
+    if overlap:   # the index kernel runs on a second stream beside the pooling of v and the compressed attention
+        spans["pool+compressed_topk (two streams)"] = ("start", "select")
+    else:
+        spans["pool"] = ("start", "pooled")
+        spans["compressed_topk"] = ("pooled", "select")
+    if fused:
+        spans["select_merge"] = ("select", "end")
+    else:
+        spans["select"] = ("select", "merge")
+        spans["merge"] = ("merge", "end")
+    per = {name: [e[a].elapsed_time(e[b]) for e in evs] for name, (a, b) in spans.items()}
+    return {"ms_per_step": wall * 1e3 / steps, "fused": fused,
+            "mean": {k: sum(v) / len(v) for k, v in per.items()},
+            "median": {k: statistics.median(v) for k, v in per.items()}}
+
+
+def guarded(fn):
+    """An extra figure must not take the headline line down with it."""
+    try:
+        return fn()
+    except Exception as exc:  # noqa: BLE001
+        return {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
+
+def _loop_ms(fn, iters=30, settle=20):
+    import torch
+
+    for _ in range(settle):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def hbm_bound_kernels(qd, kd, vd, gd, block, es):
+    """GB/s of the memory-bound kernels, each alone on one stream, from their algorithmic bytes: pooling of one tensor,
+    the layer's one pass over the packed projection, LayerNorm + RoPE of one tensor, the standalone merge."""
+    import torch
+
+    import speed3r_amd as s3r
+    from speed3r_amd.layers import RoPE2D
+    from speed3r_amd.sparse_attn import ops
+
+    _, h, n, d = qd.shape
+    nc = -(-n // block)
+    out = {}
+    with torch.no_grad():
+        ms = _loop_ms(lambda: s3r.pool_mean(qd, block))
+        out["pool"] = (n + nc) * h * d * es / (ms * 1e-3) / 1e9
+        out["pool_ms_per_tensor"] = ms
+        prepass = _prepass_stage(qd, kd, vd, block)
+        ms = _loop_ms(prepass)
+        out["prepass"] = ((3 + 2) * n * h * d * es + 3 * nc * h * d * es + n * 2 * 8) / (ms * 1e-3) / 1e9
+        out["prepass_ms"] = ms
+        del prepass
+        t = torch.arange(n, device=qd.device) % 1041
+        patch = (t - 5).clamp(min=0)
+        pos = torch.where((t >= 5)[:, None], torch.stack((patch // 28 + 1, patch % 28 + 1), dim=-1), torch.zeros_like(t)[:, None])[None]
+        cos, sin = RoPE2D(100.0).tables(64, 39, qd.device, qd.dtype)
+        w = torch.ones(64, dtype=qd.dtype, device=qd.device)
+        ms = _loop_ms(lambda: ops.norm_rope(qd, pos, cos, sin, w, w, 1e-6))
+        out["norm_rope"] = 2 * n * h * d * es / (ms * 1e-3) / 1e9
+        out["norm_rope_ms"] = ms
+        o_cmp = s3r.pool_mean(vd, block)
+        ms = _loop_ms(lambda: s3r.gated_merge(o_cmp, vd, gd, block))
+        out["merge"] = (2 * n * h * d + n * h * 2 + nc * h * d) * es / (ms * 1e-3) / 1e9
+        out["merge_ms"] = ms
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_cfg4(args):
+    """The 1000-frame layer (1 041 000 tokens, top-k 16) from the same generator drawn on the device: ms per layer, the
+    selection kernel's share of the bf16 MFMA peak and the peak footprint."""
+    import torch
+
+    import speed3r_amd as s3r
+    from speed3r_amd import workloads
+
+    dev = torch.device("cuda:0")
+    cfg = workloads.CONFIGS["cfg4"]
+    qd, kd, vd = workloads.make_qkv_on_device(cfg.frames, cfg.dtype, cfg.seed, cfg.low_rank, dev)
+    gd = torch.sigmoid(torch.randn((1, 16, cfg.tokens, 2), device=dev, generator=torch.Generator(device=dev).manual_seed(cfg.seed + 1000))).to(cfg.dtype)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+
+    def step(timeline=None):
+        return s3r.sparse_global_attention(qd, kd, vd, gd, 64, cfg.topk, timeline=timeline)
+
+    global SETTLE_STEPS
+    keep, SETTLE_STEPS = SETTLE_STEPS, 10
+    try:
+        t = time_layer(step, 10, 0, True, True)
+    finally:
+        SETTLE_STEPS = keep
+    sel = t["mean"]["select_merge"]
+    res = {"workload": f"{cfg.name}: {cfg.tokens} tokens, 16 heads x 64, block 64, top-k {cfg.topk}, drawn on the device",
+           "ms_per_layer": t["ms_per_step"], "kernels_ms": t["mean"], "steps": 10, "settle_steps": 10,
+           "select_merge_frac_of_mfma_peak": workloads.selection_flops(cfg.tokens, cfg.topk) / (sel * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+           "effective_tflops": (workloads.selection_flops(cfg.tokens, cfg.topk) + workloads.compressed_flops(cfg.tokens)) / (t["ms_per_step"] * 1e-3) / 1e12,
+           "peak_mem_gb": torch.cuda.max_memory_allocated() / 1e9}
+    del qd, kd, vd, gd
+    torch.cuda.empty_cache()
+    return res
 
 
 def run_backward(args, cfg, qd, kd, vd, block, topk) -> int:
@@ -251,7 +392,8 @@ def main() -> int:
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     if args.config == "cfg5":
-        return run_end_to_end(args)
+        print(json.dumps(run_end_to_end(args)))
+        return 0
     dev = torch.device("cuda:0")
     cfg, q, k, v, gate = workloads.make_config(args.config)
     topk = args.topk or cfg.topk
@@ -293,35 +435,12 @@ def main() -> int:
             print(f"{args.only}: {(time.perf_counter() - t0) * 1e3 / args.steps:.4f} ms per launch", file=sys.stderr)
         return 0
 
-    with torch.no_grad():
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        evs = [{} for _ in range(args.steps)]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(evs[i])
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        peak_mem = torch.cuda.max_memory_allocated()
-
-    ms_per_step = wall * 1e3 / args.steps
+    torch.cuda.reset_peak_memory_stats()
+    t = time_layer(step, args.steps, args.warmup, overlap, fused)
+    peak_mem = torch.cuda.max_memory_allocated()
+    ms_per_step, kern_ms, kern_med, fused = t["ms_per_step"], t["mean"], t["median"], t["fused"]
     nc = -(-n // block)
-    def span(a, b):
-        return sum(e[a].elapsed_time(e[b]) for e in evs) / args.steps
-
-    fused = fused and "merge" not in evs[0]   # the merge runs in the selection kernel's epilogue only where that is built
     sel_name = "select_merge" if fused else "select"
-    if overlap:   # the index kernel runs on a second stream beside the pooling of v and the compressed attention
-        kern_ms = {"pool+compressed_topk (two streams)": span("start", "select")}
-    else:
-        kern_ms = {"pool": span("start", "pooled"), "compressed_topk": span("pooled", "select")}
-    if fused:
-        kern_ms["select_merge"] = span("select", "end")
-    else:
-        kern_ms["select"] = span("select", "merge")
-        kern_ms["merge"] = span("merge", "end")
     f_sel = workloads.selection_flops(n, topk, block=block)
     f_cmp = workloads.compressed_flops(n, block=block)
     sel_tflops = f_sel / (kern_ms[sel_name] * 1e-3) / 1e12
@@ -336,6 +455,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_steps": SETTLE_STEPS,
         "ms_per_step": ms_per_step,
         "higher_is_better": False,
         "scaling": "weak",
@@ -350,6 +470,7 @@ def main() -> int:
         },
         "effective_tflops": (f_sel + f_cmp) / (ms_per_step * 1e-3) / 1e12,
         "kernels_ms": kern_ms,
+        "kernels_median_ms": kern_med,
         "hbm_gbs": {**({} if overlap else {"pool": pool_bytes / (kern_ms["pool"] * 1e-3) / 1e9}),
                     **({} if fused else {"merge": merge_bytes / (kern_ms["merge"] * 1e-3) / 1e9})},
         "peak_mem_gb": peak_mem / 1e9,
@@ -360,12 +481,27 @@ def main() -> int:
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": sel_tflops / PEAK_BF16_TFLOPS,
+            "frac_of_median_launch": f_sel / (kern_med[sel_name] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
             # HBM bytes per launch: not measured inside this run; the figure is the one rocprofv3 FETCH_SIZE / WRITE_SIZE
-            # gave for this kernel on this workload, scaled by a plain copy (file named in traffic_source)
+            # gave for this kernel on this workload, scaled by a plain copy (file named in traffic_source, which also
+            # names the commit of the kernel it was measured on)
             "traffic": MEASURED_TRAFFIC.get((args.config, topk, block, fused), (None, None))[0],
             "traffic_source": MEASURED_TRAFFIC.get((args.config, topk, block, fused), (None, None))[1],
         },
     }
+    headline = args.config == "cfg3" and block == 64 and topk == 16 and not args.no_extras
+    if headline:
+        t_extras = time.perf_counter()
+        result["hbm_gbs"].update(guarded(lambda: hbm_bound_kernels(qd, kd, vd, gd, block, es)))
+        del qd, kd, vd, gd
+        torch.cuda.empty_cache()
+        result["cfg4"] = guarded(lambda: run_cfg4(args))
+        if time.perf_counter() - t_extras < 240:
+            result["cfg5"] = guarded(lambda: {k2: v2 for k2, v2 in run_end_to_end(args, steps=3, warmup=2).items()
+                                              if k2 in ("value", "unit", "ms_per_step", "sparse_attention_share",
+                                                        "sparse_attention_ms_per_layer", "peak_mem_gb", "steps", "warmup")})
+            if "value" in result["cfg5"]:
+                result["cfg5"]["frames_per_s"] = result["cfg5"].pop("value")
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v, gate, block, topk, args.cpu_heads)
     print(json.dumps(result))

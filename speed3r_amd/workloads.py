@@ -73,6 +73,30 @@ def make_qkv(frames: int, dtype: torch.dtype, seed: int, low_rank: bool, heads: 
     return tuple(out)
 
 
+def make_qkv_on_device(frames: int, dtype: torch.dtype, seed: int, low_rank: bool, device, heads: int = HEADS,
+                       head_dim: int = HEAD_DIM, tokens_per_frame: int = TOKENS_PER_FRAME):
+    """The generator of :func:`make_qkv` drawn on ``device`` from that device's own seeded stream: the same
+    distribution (noise plus per-frame low-rank component), other bits.  For timing runs that need no CPU checker."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    n = frames * tokens_per_frame
+    out = []
+    if low_rank:
+        rank = 8
+        w = torch.randn((heads, rank, head_dim), generator=g, device=device) / rank ** 0.5
+        u_qk = torch.bmm(torch.randn((heads, frames, rank), generator=g, device=device) * 0.5, w)
+        u_v = torch.bmm(torch.randn((heads, frames, rank), generator=g, device=device) * 0.5, w)
+    for which in range(3):
+        t = torch.empty((1, heads, n, head_dim), dtype=dtype, device=device)
+        for h in range(heads):   # one head at a time: the fp32 draw of a whole tensor would double the footprint
+            x = torch.randn((n, head_dim), generator=g, device=device) / 8.0
+            if low_rank:
+                u = (u_v if which == 2 else u_qk)[h]
+                x = (x.view(frames, tokens_per_frame, head_dim) + u[:, None, :]).view(n, head_dim)
+            t[0, h] = x.to(dtype)
+        out.append(t)
+    return tuple(out)
+
+
 def make_gate(n: int, dtype: torch.dtype, seed: int, heads: int = HEADS) -> torch.Tensor:
     """Gate ``[1, heads, n, 2] = sigmoid(N(0,1))`` from its own seeded stream."""
     g = torch.Generator().manual_seed(seed + 1000)
