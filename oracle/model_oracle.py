@@ -6,7 +6,9 @@ TEST INFRASTRUCTURE ONLY -- never imported by the product package.
 The model follows the reference's structure (pi3/models/pi3_sparse.py:214-321: encoder -> alternating frame-local /
 global decoder blocks -> point, confidence and camera decoders and heads; pi3/models/layers/block.py:259-335: pre-norm
 block with LayerScale; pi3/models/layers/attention.py:324-348: dense attention with qk-norm and RoPE) with the Pi3
-teacher's token layout (register tokens, then patches in row-major order).  Here every piece is a library routine on
+teacher's token layout (register tokens, then patches in row-major order) or, with ``tile > 0``, with the reference
+model's own one (no register tokens, positions from 0, patches of a frame in tile-major order through the decoder and
+back in row-major order in front of the heads: pi3_sparse.py:29-71,163-169,228-229,265-269).  Here every piece is a library routine on
 the parameters of a ``state_dict``: ``F.conv2d`` for the patch embedding, ``F.layer_norm``, ``F.linear``, ``F.gelu``,
 ``F.scaled_dot_product_attention`` for the frame-local attentions, ``rope2d`` and ``sparse_layer`` of this package
 (both pinned on their own) for the rotary embedding and the global blocks, ``F.pixel_shuffle`` for the dense heads.
@@ -54,9 +56,25 @@ def _count(sd, prefix):
     return 1 + max(int(k[len(prefix):].split(".")[0]) for k in sd if k.startswith(prefix))
 
 
+def tile_major_index(gh: int, gw: int, tile: int) -> torch.Tensor:
+    """``perm[i]`` = row-major index of the token that stands at place ``i`` of the tile-major order: place
+    ``((ty * (gw // tile) + tx) * tile + py) * tile + px`` holds token ``(ty * tile + py, tx * tile + px)``
+    (pi3_sparse.py:29-45, 'b (nh ph) (nw pw) d -> b (nh nw ph pw) d')."""
+    perm = torch.empty(gh * gw, dtype=torch.long)
+    i = 0
+    for ty in range(gh // tile):
+        for tx in range(gw // tile):
+            for py in range(tile):
+                for px in range(tile):
+                    perm[i] = (ty * tile + py) * gw + tx * tile + px
+                    i += 1
+    return perm
+
+
 def pi3_sparse_like_forward(sd: dict, imgs: torch.Tensor, heads: int, patch: int, block_tokens: int, topk: int,
-                            rope_base: float = 100.0, return_features: bool = False) -> dict:
-    """imgs ``[B,F,3,H,W]`` in [0,1], ``sd`` the model's state dict as fp32 CPU tensors -> the model's outputs."""
+                            rope_base: float = 100.0, return_features: bool = False, tile: int = 0) -> dict:
+    """imgs ``[B,F,3,H,W]`` in [0,1], ``sd`` the model's state dict as fp32 CPU tensors -> the model's outputs.
+    ``tile > 0``: the reference model's token pipeline (no register tokens allowed in ``sd``)."""
     sd = {k: v.detach().float().cpu() for k, v in sd.items()}
     b, f, _, hh, ww = imgs.shape
     gh, gw = hh // patch, ww // patch
@@ -76,8 +94,16 @@ def pi3_sparse_like_forward(sd: dict, imgs: torch.Tensor, heads: int, patch: int
     x = torch.cat((sd["register_token"].expand(b * f, -1, -1), x), dim=1)
     t = x.shape[1]
     yy, xx = torch.meshgrid(torch.arange(gh), torch.arange(gw), indexing="ij")
-    pos = torch.cat((torch.zeros((nreg, 2), dtype=torch.long), torch.stack((yy, xx), dim=-1).reshape(-1, 2) + 1), dim=0)
+    if tile:
+        assert nreg == 0 and gh % tile == 0 and gw % tile == 0
+        pos = torch.stack((yy, xx), dim=-1).reshape(-1, 2)
+    else:
+        pos = torch.cat((torch.zeros((nreg, 2), dtype=torch.long), torch.stack((yy, xx), dim=-1).reshape(-1, 2) + 1), dim=0)
     pos = pos[None].expand(b * f, -1, -1).contiguous()
+    pos_rows = pos                                    # what the head decoders see
+    if tile:                                          # decoder: a frame's tokens and positions gathered into tile-major order
+        perm = tile_major_index(gh, gw, tile)
+        x, pos = x[:, perm], pos[:, perm]
     local_out = None
     for i in range(_count(sd, "local_decoder.")):
         pre = f"local_decoder.{i}"
@@ -95,6 +121,10 @@ def pi3_sparse_like_forward(sd: dict, imgs: torch.Tensor, heads: int, patch: int
 
         x = _block(x, sd, pre, global_attention, True)
     feat = torch.cat((local_out, x), dim=-1)
+    if tile:                                          # back: the token at tile-major place i returns to row-major place perm[i]
+        back = torch.empty_like(feat)
+        back[:, perm] = feat
+        feat, pos = back, pos_rows
 
     def head_decoder(name):
         y = F.linear(feat, sd[name + ".project.weight"], sd[name + ".project.bias"])

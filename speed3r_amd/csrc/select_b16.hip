@@ -439,9 +439,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       }
     };
     // Two of the unit's 16 exponentials per slot (8 slots).  A slot computes its pair and rounds / sums the pair of the
-    // slot before, so that no instruction waits on an exponential just issued.  Row sums over the ROUNDED
-    // probabilities: with a reference below the maximum a probability is not a power of two, and its rounding cancels
-    // in p / sum p only if the sum has it too.
+    // slot before, so that no instruction waits on an exponential just issued.  Row sums over the unrounded
+    // probabilities (two additions; the dot product of the rounded pair with ones is the slower instruction here).
     float px0 = 0.f, px1 = 0.f;  // the pair in flight
     auto exps_finish = [&](auto qt_tag, auto j_tag) {
       constexpr int QT = decltype(qt_tag)::value;
@@ -451,7 +450,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       pk[1] = (E)px1;
       pf[QT][jj][e8] = pk[0];
       pf[QT][jj][e8 + 1] = pk[1];
-      l_i[QT] = Mma<E>::dot_ones(pk, l_i[QT]);
+      l_i[QT] += px0 + px1;
     };
     auto exps = [&](auto qt_tag, auto j_tag) {
       constexpr int QT = decltype(qt_tag)::value;
@@ -594,7 +593,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
         });
         exact = was_exact;
       }
-      const float big = 1.2676506e30f;  // 2^100
+      // the sums add the unrounded fp32 probabilities (all >= 0): a sum below the bound proves that every probability
+      // was below it when it was rounded; fp16 ends at 65504, bf16 has fp32's range (2^100 leaves room for the products)
+      const float big = std::is_same<E, f16_t>::value ? 65504.f : 1.2676506e30f;
       if (exact || !__any(!(l_i[0] < big) || !(l_i[1] < big))) break;
       // rare: some reference was far too low; start over with the running maximum
 #pragma unroll

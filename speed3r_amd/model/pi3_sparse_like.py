@@ -15,6 +15,11 @@ pi3/models/layers/transformer_head.py (head decoders, linear pixel-shuffle head)
   flat sequence in blocks of 64 tokens with the ragged-tail policy of the kernels;
 * heads: three 5-block frame-local decoders on the concatenated outputs of the last local and global blocks, a linear
   pixel-shuffle head for local points and confidence, a small pose head.
+* ``token_order="tile"`` with ``num_register=0, block_tokens=16, topk=32`` is the reference model's own token
+  pipeline: no register tokens (pi3_sparse.py:163-169), positions from 0 (pos_embed.py:162-174), every frame's patches
+  in 4 x 4-tile-major order through the decoder (pi3_sparse.py:29-45,228-229) and back in row-major order in front of
+  the head decoders (:265-269), global attention over 16-token blocks = 4 x 4 patch tiles with the 32 best blocks
+  (sparse_attention.py:73,98,112).  The patch grid must split into 4 x 4 tiles (frames of 56-pixel multiples).
 
 All dense GEMMs are library calls (torch on rocBLAS/hipBLASLt); the frame-local dense attentions run on the package's
 dense flash kernel (the one behind the compressed branch) for bf16/fp16 inference with head_dim 64, else on
@@ -33,6 +38,7 @@ from torch import Tensor, nn
 from ..layers import RoPE2D, SparseFlashAttentionRope
 from ..layers.sparse_attention import norm_rope_fused_or_eager
 from ..sparse_attn import ops
+from .token_order import tile_major, tile_major_inverse
 
 
 class Mlp(nn.Module):
@@ -201,9 +207,13 @@ class PoseHead(nn.Module):
 
 class Pi3SparseLike(nn.Module):
     def __init__(self, dim=1024, enc_depth=24, dec_depth=36, num_heads=16, head_depth=5, patch=14, grid=(37, 28),
-                 num_register=5, block_tokens=64, topk=16, rope_freq=100.0) -> None:
+                 num_register=5, block_tokens=64, topk=16, rope_freq=100.0, token_order="row", tile=4) -> None:
         super().__init__()
         assert dec_depth % 2 == 0 and int(block_tokens ** 0.5) ** 2 == block_tokens
+        assert token_order in ("row", "tile")
+        assert token_order == "row" or num_register == 0, "the tile-major order has no place for register tokens"
+        self.token_order = token_order
+        self.tile = tile
         self.patch = patch
         self.encoder = PatchEncoder(dim, enc_depth, num_heads, patch, grid)
         self.rope = RoPE2D(freq=rope_freq, max_positions=max(grid) + 2)
@@ -226,9 +236,11 @@ class Pi3SparseLike(nn.Module):
 
     def _positions(self, f: int, gh: int, gw: int, device) -> Tensor:
         yy, xx = torch.meshgrid(torch.arange(gh, device=device), torch.arange(gw, device=device), indexing="ij")
-        patch = torch.stack((yy, xx), dim=-1).reshape(gh * gw, 2) + 1           # register tokens sit at (0, 0)
-        reg = torch.zeros((self.register_token.shape[1], 2), dtype=patch.dtype, device=device)
-        return torch.cat((reg, patch), dim=0)[None].expand(f, -1, -1).contiguous()
+        patch = torch.stack((yy, xx), dim=-1).reshape(gh * gw, 2)
+        if self.register_token.shape[1] == 0:                                     # the reference model: positions from 0
+            return patch[None].expand(f, -1, -1).contiguous()
+        reg = torch.zeros((self.register_token.shape[1], 2), dtype=patch.dtype, device=device)   # register tokens sit at (0, 0)
+        return torch.cat((reg, patch + 1), dim=0)[None].expand(f, -1, -1).contiguous()
 
     def forward(self, imgs: Tensor, return_features: bool = False) -> dict:
         """imgs [B, F, 3, H, W] in [0,1] -> dict(points, local_points, conf, camera_poses); ``return_features`` adds the
@@ -243,12 +255,19 @@ class Pi3SparseLike(nn.Module):
         x = torch.cat((self.register_token.expand(b * f, -1, -1), x), dim=1)       # [B*F, T, dim]
         t = x.shape[1]
         pos = self._positions(b * f, gh, gw, x.device)                             # [B*F, T, 2]
+        tiled = self.token_order == "tile"
+        if tiled:                                                                  # tokens and their positions, tile-major
+            x, pos_dec = tile_major(x, gh, gw, self.tile), tile_major(pos, gh, gw, self.tile)
+        else:
+            pos_dec = pos
         local_out = None
         for local_blk, global_blk in zip(self.local_decoder, self.global_decoder):
-            x = local_blk(x, xpos=pos)
+            x = local_blk(x, xpos=pos_dec)
             local_out = x
-            x = global_blk(x.reshape(b, f * t, -1), xpos=pos.reshape(b, f * t, 2)).reshape(b * f, t, -1)
+            x = global_blk(x.reshape(b, f * t, -1), xpos=pos_dec.reshape(b, f * t, 2)).reshape(b * f, t, -1)
         feat = torch.cat((local_out, x), dim=-1)
+        if tiled:                                                                  # the heads see row-major tokens again
+            feat = tile_major_inverse(feat, gh, gw, self.tile)
         nreg = self.register_token.shape[1]
         pts = self.point_head(self.point_decoder(feat, pos)[:, nreg:], gh, gw).float()
         conf = self.conf_head(self.conf_decoder(feat, pos)[:, nreg:], gh, gw).float()

@@ -63,9 +63,10 @@ def test_dense_attention_into_a_caller_view():
     assert torch.equal(buf.permute(0, 2, 1, 3), ref)
 
 
-def _randomised_small_model(seed=0):
+def _randomised_small_model(seed=0, **kw):
     torch.manual_seed(seed)
-    m = Pi3SparseLike(dim=128, enc_depth=2, dec_depth=4, num_heads=2, head_depth=1, grid=(4, 6), block_tokens=16, topk=4)
+    m = Pi3SparseLike(dim=128, enc_depth=2, dec_depth=4, num_heads=2, head_depth=1, block_tokens=16, topk=4,
+                      **{"grid": (4, 6), **kw})
     with torch.no_grad():                      # non-trivial values where the constructors put zeros or near-zeros
         for name, p in m.named_parameters():
             if name.endswith("gamma"):
@@ -115,6 +116,40 @@ def test_small_model_bf16_stays_close_to_the_fp32_restatement():
         assert rel <= bar, (key, rel)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_small_model_in_the_reference_token_order(dtype):
+    """The reference model's own setting in small: no register tokens, positions from 0, 4 x 4-tile-major token order
+    through the decoder (pi3_sparse.py:29-71,228-229,265-269), 16-token blocks = one tile each, against the restatement
+    extended the same way (a gather index built by plain loops).  12 frames of 8 x 12 patches = 1152 tokens = 72 blocks,
+    top-8.  fp32: 1e-4 of each output's scale; bf16: relative L2 error at most 2 % (near-ties in a selection may flip)."""
+    torch.manual_seed(6)
+    m = Pi3SparseLike(dim=128, enc_depth=2, dec_depth=4, num_heads=2, head_depth=1, grid=(8, 12), block_tokens=16, topk=8,
+                      num_register=0, token_order="tile")
+    with torch.no_grad():
+        for name, p in m.named_parameters():
+            if name.endswith("gamma"):
+                p.copy_(0.5 + 0.5 * torch.rand_like(p))
+            elif "gate.0" in name or name.endswith("cls_token") or name.endswith("register_tokens"):
+                p.copy_(0.3 * torch.randn_like(p))
+            elif name.endswith(".bias"):
+                p.copy_(0.1 * torch.randn_like(p))
+    m = m.eval().to(dtype)
+    frames, hh, ww = 12, 112, 168
+    imgs = torch.rand((1, frames, 3, hh, ww), generator=torch.Generator().manual_seed(7))
+    want = oracle.pi3_sparse_like_forward(m.state_dict(), imgs, heads=2, patch=14, block_tokens=16, topk=8,
+                                          return_features=True, tile=4)
+    m = m.to(DEV)
+    with torch.no_grad():
+        got = m(imgs.to(DEV), return_features=True)
+    assert all(b.attn.last_path in ("fused-merge", "two-operators") for b in m.global_decoder)
+    for key in want:
+        g, w = got[key].float().cpu(), want[key]
+        if dtype == torch.float32:
+            assert (g - w).abs().max().item() <= 1e-4 * max(1.0, w.abs().max().item()), key
+        else:
+            assert ((g - w).norm() / w.norm()).item() <= 0.02, key
+
+
 def test_rope_tables_follow_the_frame_size():
     """Frames larger than the grid the model was built for: the fused norm/RoPE kernel's tables are sized from the
     call (positions beyond a table would be clamped): the model's dense attention with RoPE on a 45-wide position range
@@ -155,6 +190,29 @@ def test_end_to_end_workload_100_frames_518x392():
     assert len(m.global_decoder) == 18 and all(b.attn.last_path == "fused-merge" for b in m.global_decoder)
     assert out["points"].shape == (1, frames, 518, 392, 3) and out["conf"].shape == (1, frames, 518, 392, 1)
     assert out["camera_poses"].shape == (1, frames, 4, 4)
+    for v in out.values():
+        assert torch.isfinite(v).all()
+    rot = out["camera_poses"][0, :, :3, :3].double()
+    assert torch.allclose(rot @ rot.transpose(-1, -2), torch.eye(3, dtype=torch.float64, device=DEV).expand(frames, 3, 3), atol=1e-4)
+    del m, out
+    torch.cuda.empty_cache()
+
+
+def test_end_to_end_workload_in_the_reference_setting_100_frames_504x392():
+    """The reference model's own setting at full size, once: 100 frames of 504 x 392 (a multiple of 56: 36 x 28 patches
+    = 63 tiles of 4 x 4, 100 800 tokens), no register tokens, tile-major order, 16-token blocks, top-32
+    (sparse_attention.py:73,98,112).  Shapes, finiteness, orthonormal rotations, all 18 global blocks on the fused route."""
+    torch.manual_seed(4)
+    with torch.device(DEV):
+        m = Pi3SparseLike(grid=(36, 28), num_register=0, token_order="tile", block_tokens=16, topk=32)
+    m = m.to(torch.bfloat16).eval()
+    frames = 100
+    imgs = torch.rand((1, frames, 3, 504, 392), generator=torch.Generator().manual_seed(4)).to(DEV)
+    with torch.no_grad():
+        out = m(imgs)
+    torch.cuda.synchronize()
+    assert len(m.global_decoder) == 18 and all(b.attn.last_path == "fused-merge" for b in m.global_decoder)
+    assert out["points"].shape == (1, frames, 504, 392, 3) and out["camera_poses"].shape == (1, frames, 4, 4)
     for v in out.values():
         assert torch.isfinite(v).all()
     rot = out["camera_poses"][0, :, :3, :3].double()

@@ -10,9 +10,10 @@ import oracle
 from speed3r_amd.model import Pi3SparseLike
 
 
-def _small_model(seed=0):
+def _small_model(seed=0, **kw):
     torch.manual_seed(seed)
-    m = Pi3SparseLike(dim=128, enc_depth=2, dec_depth=4, num_heads=2, head_depth=1, grid=(4, 6), block_tokens=16, topk=4)
+    m = Pi3SparseLike(dim=128, enc_depth=2, dec_depth=4, num_heads=2, head_depth=1, block_tokens=16, topk=4,
+                      **{"grid": (4, 6), **kw})
     with torch.no_grad():                      # non-trivial values where the constructors put zeros or near-zeros
         for name, p in m.named_parameters():
             if name.endswith("gamma"):
@@ -70,3 +71,23 @@ def test_restatement_reacts_to_every_parameter_group():
         sd2[name] = sd[name] + 0.05 * torch.randn(sd[name].shape, generator=torch.Generator().manual_seed(3))
         out = oracle.pi3_sparse_like_forward(sd2, imgs, heads=2, patch=14, block_tokens=16, topk=4, return_features=True)
         assert any((out[k] - base[k]).abs().max().item() > 1e-6 for k in base), name
+
+
+def test_restatement_in_the_reference_token_order():
+    """The reference model's own token pipeline (no register tokens, positions from 0, 4 x 4-tile-major order through
+    the decoder and row-major order again in front of the heads): the package's modules reorder with reshape/permute,
+    the restatement with a gather index built by plain loops.  8 x 8 patches per frame = 4 tiles = four 16-token blocks."""
+    m = _with_oracle_layers(_small_model(2, grid=(8, 8), num_register=0, token_order="tile"))
+    frames, hh, ww = 3, 112, 112
+    imgs = torch.rand((1, frames, 3, hh, ww), generator=torch.Generator().manual_seed(5))
+    with torch.no_grad():
+        got = m(imgs, return_features=True)
+        want = oracle.pi3_sparse_like_forward(m.state_dict(), imgs, heads=2, patch=14, block_tokens=16, topk=4,
+                                              return_features=True, tile=4)
+        row = oracle.pi3_sparse_like_forward(m.state_dict(), imgs, heads=2, patch=14, block_tokens=16, topk=4, return_features=True)
+    for key in want:
+        assert got[key].shape == want[key].shape, key
+        scale = max(1.0, want[key].abs().max().item())
+        assert (got[key].float() - want[key]).abs().max().item() <= 2e-4 * scale, key
+    # the order matters: the same weights on row-major tokens (blocks = runs of 16 tokens of a patch row pair) differ
+    assert (row["features"] - want["features"]).abs().max().item() > 1e-3
