@@ -37,7 +37,8 @@ typedef std::integral_constant<int, 0> H0;
 typedef std::integral_constant<int, 1> H1;
 
 // UNION: the wave walks the union of its four lists, see below (default); otherwise pairs of list entries.
-template <typename E, bool UNION>
+// WIDE (union walk): K or V rows lie 4 GiB or more behind the tensor's first row (beyond a 32-bit byte offset).
+template <typename E, bool UNION, bool WIDE>
 __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p, int nqb, int ngrp, int nwg_per_bh, int total_wg) {
   typedef typename Mma<E>::V8 V8;
   typedef typename Mma<E>::V2 V2;
@@ -317,7 +318,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       cb = (uint32_t)__builtin_amdgcn_readfirstlane(v.w);
     };
 
-    // ---- transfers: one descriptor per tensor, the block's byte offset rides in the scalar offset ----
+    // ---- transfers: one descriptor per block, based at the block's first row (a 64-bit address: byte offsets inside
+    // the instruction stay below 16 rows, whatever the row stride and the sequence length) ----
     // (the K swizzle of a block's rows 8..15 differs from that of its rows 0..7: one offset per instruction of a block)
     const uint32_t koff = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ k_swizzle(lr)) * 16);
     const uint32_t koff8 = (uint32_t)lr * krow + (uint32_t)(((lane & 7) ^ k_swizzle(lr + 8)) * 16);
@@ -327,17 +329,22 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     const LdsPtr v_lds[2] = {(LdsPtr)lds_v0 + wave * kHalfBytes, (LdsPtr)lds_v1 + wave * kHalfBytes};
     // 16 rows of one block -> 2 KB at dst.  The instruction's immediate offset moves the LDS side and the global side
     // alike; the scalar offset makes up the difference (row strides are at least 128 bytes).
-    auto dma_block = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb, int32_t blk) {
-      const uint32_t so = (uint32_t)blk * 16u * rowb;
+    // WIDE (a tensor whose last row lies 4 GiB or more behind its first): the descriptor is based at the block itself,
+    // a 64-bit address; otherwise at the tensor, and the block's byte offset rides in the 32-bit scalar offset (a
+    // multiplication less per block)
+    auto dma_block = [&](const E* base, int64_t row_elems, int32_t rec, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb, int32_t blk) {
+      const int64_t far = WIDE ? (int64_t)blk * 16 * row_elems : 0;
+      const uint32_t so = WIDE ? 0u : (uint32_t)blk * 16u * rowb;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(base + far), 0, rec, 0x00020000);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off0, so, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, off8, so + (8u * rowb - 1024u), 1024, 0);
     };
-    auto dma_ragged = [&](const __amdgpu_buffer_rsrc_t& rs, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb) {  // rows beyond the sequence re-read its last row
-      const uint32_t so = (uint32_t)ragged_blk * 16u * rowb;
+    auto dma_ragged = [&](const E* base, int64_t row_elems, LdsPtr dst, uint32_t off0, uint32_t off8, uint32_t rowb) {  // rows beyond the sequence re-read its last row
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)ragged_blk * 16 * row_elems), 0, -1, 0x00020000);
       const int r0 = lr < ragged_last ? lr : ragged_last, r1 = 8 + lr < ragged_last ? 8 + lr : ragged_last;
       const uint32_t col0 = off0 - (uint32_t)lr * rowb, col8 = off8 - (uint32_t)lr * rowb;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (uint32_t)r0 * rowb + col0, so, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst + 1024, 16, (uint32_t)r1 * rowb + col8, so, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (uint32_t)r0 * rowb + col0, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst + 1024, 16, (uint32_t)r1 * rowb + col8, 0, 0, 0);
     };
     // A tile beyond the end of the list (a < 0) is requested all the same, through a descriptor of zero records:
     // every lane is out of range, nothing is fetched, and the count of outstanding transfers does not depend on the
@@ -349,18 +356,16 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
     };
     auto dma_k = [&](auto par_tag, int32_t a, int32_t b2) {
       constexpr int P = decltype(par_tag)::value;
-      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, records(a), 0x00020000);
-      dma_block(rs, k_lds[P], koff, koff8, krow, a);
-      dma_block(rs, k_lds[P] + 2048, koff, koff8, krow, b2 < 0 ? a : b2);
+      const int32_t rec = records(a);
+      dma_block(kp, p.skn, rec, k_lds[P], koff, koff8, krow, a);
+      dma_block(kp, p.skn, rec, k_lds[P] + 2048, koff, koff8, krow, b2 < 0 ? a : b2);
     };
     auto dma_v = [&](auto par_tag, int32_t a, int32_t b2) {
       constexpr int P = decltype(par_tag)::value;
-      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, records(a), 0x00020000);
-      dma_block(rs, v_lds[P], voff, voff, vrow, a);
-      dma_block(rs, v_lds[P] + 2048, voff, voff, vrow, b2 < 0 ? a : b2);
+      const int32_t rec = records(a);
+      dma_block(vp, p.svn, rec, v_lds[P], voff, voff, vrow, a);
+      dma_block(vp, p.svn, rec, v_lds[P] + 2048, voff, voff, vrow, b2 < 0 ? a : b2);
     };
-    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, -1, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, -1, 0x00020000);
     V8 ak[4];       // K fragments of one tile
     V8 vfr[2][2];   // V^T fragments of one tile [jj][dt]
     auto load_k = [&](auto par_tag) {
@@ -571,10 +576,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void select_b16_kernel(AttnParams p
       }
       if (ragged_cnts != 0) {  // the block that ends the sequence early: one unpipelined step with the running maximum
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): earlier reads of the buffers are done
-        dma_ragged(rk, k_lds[0], koff, koff8, krow);
-        dma_ragged(rk, k_lds[0] + 2048, koff, koff8, krow);  // the tile's second block: the same rows again (finite values)
-        dma_ragged(rv, v_lds[0], voff, voff, vrow);
-        dma_ragged(rv, v_lds[0] + 2048, voff, voff, vrow);
+        dma_ragged(kp, p.skn, k_lds[0], koff, koff8, krow);
+        dma_ragged(kp, p.skn, k_lds[0] + 2048, koff, koff8, krow);  // the tile's second block: the same rows again (finite values)
+        dma_ragged(vp, p.svn, v_lds[0], voff, voff, vrow);
+        dma_ragged(vp, p.svn, v_lds[0] + 2048, voff, voff, vrow);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         load_k(H0{});
         load_v(H0{});
@@ -703,15 +708,17 @@ int launch_select_b16(const AttnParams& p, int dtype, void* stream) {
     const char* e = getenv("S3R_B16_KERNEL");
     return e != nullptr && strcmp(e, "pairs") == 0;
   }();
-  // the union walk addresses a head's K and V rows through 32-bit byte offsets from one descriptor per tensor
+  // 32-bit byte offsets inside a transfer instruction span 16 rows of a block
+  if (16 * p.skn * 2 + 128 > 0xffffffffLL || 16 * p.svn * 2 + 128 > 0xffffffffLL)
+    return fail(S3R_ERR_UNSUPPORTED, "s3r_select_attn, 16-token blocks: row stride too large");
+  const bool pairs = pairs_env;
   const int64_t es = 2;
-  const bool wide = (p.Lq - 1) * p.skn * es + 128 > 0xffffffffLL || (p.Lq - 1) * p.svn * es + 128 > 0xffffffffLL;
-  const bool pairs = pairs_env || wide;
-#define S3R_B16(E, U) hipLaunchKernelGGL((b16::select_b16_kernel<E, U>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total)
+  const int wide = (p.Lq - 1) * p.skn * es + 128 > 0xffffffffLL || (p.Lq - 1) * p.svn * es + 128 > 0xffffffffLL;
+#define S3R_B16(E, U, W) hipLaunchKernelGGL((b16::select_b16_kernel<E, U, W>), grid, blk, 0, st, p, (int)nqb, (int)ngrp, (int)nwg, (int)total)
   if (dtype == S3R_BF16) {
-    if (pairs) S3R_B16(bf16_t, false); else S3R_B16(bf16_t, true);
+    if (pairs) S3R_B16(bf16_t, false, false); else if (wide) S3R_B16(bf16_t, true, true); else S3R_B16(bf16_t, true, false);
   } else {
-    if (pairs) S3R_B16(f16_t, false); else S3R_B16(f16_t, true);
+    if (pairs) S3R_B16(f16_t, false, false); else if (wide) S3R_B16(f16_t, true, true); else S3R_B16(f16_t, true, false);
   }
 #undef S3R_B16
   return check_launch("select_b16_kernel");

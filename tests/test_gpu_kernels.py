@@ -591,3 +591,29 @@ def test_select_with_a_query_row_stride_beyond_the_transfer_offsets():
     want = oracle.select_attention(q, k.cpu(), v.cpu(), idx.cpu(), 64, out_dtype=torch.float32)
     assert max_abs(s3r.select_attn(q_far, k, v, idx, 64), want) <= 2e-2
     assert max_abs(s3r.select_attn(q.to(DEV), k, v, idx, 64), want) <= 2e-2
+
+
+def test_select_block16_rows_beyond_4_gib_from_the_tensor_start():
+    """16-token blocks on K and V views whose last rows lie more than 4 GiB behind the first (row stride just below
+    2^20 elements, 2112 rows): every transfer instruction addresses its rows from a descriptor based at the block, so
+    the byte offsets stay small whatever the tensor's extent.  (The layer passes V as the in-place view of the packed
+    projection, 6 KB per row: the same holds there from 700 000 tokens on.)"""
+    n, h, kk, stride = 2112, 1, 8, (1 << 20) - 64
+    q = _randn((1, h, n, 64), 60, torch.bfloat16, 0.5)
+    k = _randn((1, h, n, 64), 61, torch.bfloat16, 0.5)
+    v = _randn((1, h, n, 64), 62, torch.bfloat16)
+    nqb = n // 16
+    idx = torch.randint(-1, nqb, (1, h, nqb, kk), generator=torch.Generator().manual_seed(63), dtype=torch.int32)
+    idx[..., 0] = nqb - 1 - torch.arange(nqb, dtype=torch.int32) % 8          # every query block reads from the far end
+    far = []
+    for t in (k, v):
+        base = torch.empty(n * stride + 64, dtype=torch.bfloat16, device=DEV)
+        view = base.as_strided((1, h, n, 64), (0, 0, stride, 1))
+        view.copy_(t)
+        far.append(view)
+    assert (n - 1) * stride * 2 > (1 << 32)
+    got = s3r.select_attn(q.to(DEV), far[0], far[1], idx.to(DEV), 16)
+    want = oracle.select_attention(q, k, v, idx, 16, out_dtype=torch.float32)
+    assert max_abs(got, want) <= 2e-2
+    del far
+    torch.cuda.empty_cache()
