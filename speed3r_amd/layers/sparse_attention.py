@@ -27,19 +27,22 @@ from ..sparse_attn.flash_attention_topk import flash_attn_topk_func
 from .pos_embed import RoPE2D, block_positions
 
 
-def norm_rope_fused_or_eager(t: Tensor, norm: nn.Module, rope, pos: Optional[Tensor]) -> Tensor:
+def norm_rope_fused_or_eager(t: Tensor, norm: nn.Module, rope, pos: Optional[Tensor], n_pos: Optional[int] = None) -> Tensor:
     """qk-norm, cast and RoPE of one ``[B,H,N,D]`` tensor (reference sparse_attention.py:103-110,120-124): one fused
     kernel where it is built -- a tensor on the GPU, head_dim 64, ``nn.Identity`` or an affine ``nn.LayerNorm`` of
     exactly that type, the package's RoPE2D or no rotation -- and the separate torch modules otherwise (any other norm
     module, a LayerNorm without affine parameters, another rope).  Same rounding points either way, except that the
-    kernel takes the LayerNorm parameters in the tokens' dtype (fp32 parameters under autocast are rounded to it)."""
+    kernel takes the LayerNorm parameters in the tokens' dtype (fp32 parameters under autocast are rounded to it).
+    ``n_pos``: number of rows of the kernel's cos/sin tables for THIS call (every coordinate in ``pos`` must be below it;
+    the kernel clamps larger ones); default: the rope module's ``max_positions``, else ``pos.max() + 1`` (a device
+    synchronisation)."""
     fused_norm = isinstance(norm, nn.Identity) or (type(norm) is nn.LayerNorm and norm.elementwise_affine)
     fused_rope = pos is None or isinstance(rope, RoPE2D)
     if t.is_cuda and t.shape[-1] == 64 and fused_norm and fused_rope and not (isinstance(norm, nn.Identity) and pos is None):
         cos = sin = None
         if pos is not None:
-            n_pos = rope.max_positions or int(pos.max()) + 1
-            cos, sin = rope.tables(64, n_pos, t.device, t.dtype)
+            rows = n_pos or rope.max_positions or int(pos.max()) + 1
+            cos, sin = rope.tables(64, rows, t.device, t.dtype)
         ln = norm if isinstance(norm, nn.LayerNorm) else None
         out = ops.norm_rope(t, pos, cos, sin, ln.weight if ln is not None else None,
                             ln.bias if ln is not None else None, ln.eps if ln is not None else 0.0)
@@ -91,10 +94,10 @@ class SparseFlashAttentionRope(nn.Module):
         self.last_prepass = None     # whether the last forward used the one-pass kernel over the packed projection
         self.last_path = None        # which route the last forward took: "fused-merge", "two-operators" or "autograd"
 
-    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
-        return norm_rope_fused_or_eager(t, norm, self.rope, pos)
+    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor], n_pos: Optional[int] = None) -> Tensor:
+        return norm_rope_fused_or_eager(t, norm, self.rope, pos, n_pos)
 
-    def _prepass(self, qkv: Tensor, h: int, block: int, pos: Optional[Tensor]):
+    def _prepass(self, qkv: Tensor, h: int, block: int, pos: Optional[Tensor], n_pos: Optional[int] = None):
         """The fused pre-pass where its conditions hold (those of ``norm_rope_fused_or_eager`` for both norms), else None."""
         def plain(norm):
             return isinstance(norm, nn.Identity) or (type(norm) is nn.LayerNorm and norm.elementwise_affine)
@@ -107,8 +110,8 @@ class SparseFlashAttentionRope(nn.Module):
             return None  # beside the norm/RoPE kernels (measured at 266 496 tokens, block 16: 10.9 against 11.2 ms per layer)
         cos = sin = None
         if pos is not None:
-            n_pos = self.rope.max_positions or int(pos.max()) + 1
-            cos, sin = self.rope.tables(64, n_pos, qkv.device, qkv.dtype)
+            rows = n_pos or self.rope.max_positions or int(pos.max()) + 1
+            cos, sin = self.rope.tables(64, rows, qkv.device, qkv.dtype)
         ln = isinstance(self.q_norm, nn.LayerNorm)
         if ln and self.q_norm.eps != self.k_norm.eps:
             return None
@@ -157,7 +160,10 @@ class SparseFlashAttentionRope(nn.Module):
         out = out.permute(0, 2, 1, 3).reshape(b, n, c)
         return self.proj_drop(self.proj(out))
 
-    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
+    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None, n_pos: Optional[int] = None) -> Tensor:
+        """``n_pos`` (optional, beyond the reference's signature): an upper bound, exclusive, of the coordinates in
+        ``xpos`` for this call; sizes the fused kernels' cos/sin tables without a device synchronisation and without
+        touching state shared between calls."""
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
             self.last_path = "autograd"
             return self._forward_with_grad(x, xpos)
@@ -174,7 +180,7 @@ class SparseFlashAttentionRope(nn.Module):
         # One pass over the packed projection: block means of the raw q, k, v (compressed branch) and norm + RoPE of
         # the full-token q and k (selection branch), each input row read once.  Where that kernel is not built
         # (head_dim other than 64, another norm or rope module): pooling kernel, then norm/RoPE per tensor.
-        pre = self._prepass(qkv, h, block, pos)
+        pre = self._prepass(qkv, h, block, pos, n_pos)
         self.last_prepass = pre is not None
         if pre is not None:
             q, k, v, q_c, k_c, v_c = pre
@@ -182,7 +188,7 @@ class SparseFlashAttentionRope(nn.Module):
             q_c, k_c, v_c = ops.pool_qkv_packed(qkv, h, block)
         # compressed branch: pooled raw projections -> norm -> RoPE at block positions -> attention + top-k
         pos_c = block_positions(xpos, block) if use_pos else None
-        q_c, k_c = self._norm_rope(q_c, self.q_norm, pos_c), self._norm_rope(k_c, self.k_norm, pos_c)
+        q_c, k_c = self._norm_rope(q_c, self.q_norm, pos_c, n_pos), self._norm_rope(k_c, self.k_norm, pos_c, n_pos)
         # the index kernel needs pooled q and k only and its result is first read by the selection kernel: where
         # it is a kernel of its own it runs on a second stream, beside the compressed attention (and the norm/RoPE of
         # the full tokens where they are separate kernels)
@@ -195,7 +201,7 @@ class SparseFlashAttentionRope(nn.Module):
 
         if pre is None:  # selection branch on strided views of the projection; norm/RoPE make q, k contiguous
             q, k, v = qkv.view(b, n, 3, h, d).permute(2, 0, 3, 1, 4).unbind(0)   # each [B, H, N, D]
-            q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
+            q, k = self._norm_rope(q, self.q_norm, pos, n_pos), self._norm_rope(k, self.k_norm, pos, n_pos)
         if side:
             join()
         if self.keep_topk_idx:

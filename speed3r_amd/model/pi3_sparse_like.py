@@ -86,15 +86,15 @@ class DenseAttentionRope(nn.Module):
         self.k_norm = norm_layer(head_dim) if qk_norm else nn.Identity()
         self.rope = rope
 
-    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor]) -> Tensor:
-        return norm_rope_fused_or_eager(t, norm, self.rope, pos)
+    def _norm_rope(self, t: Tensor, norm: nn.Module, pos: Optional[Tensor], n_pos: Optional[int] = None) -> Tensor:
+        return norm_rope_fused_or_eager(t, norm, self.rope, pos, n_pos)
 
-    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None) -> Tensor:
+    def forward(self, x: Tensor, attn_bias=None, xpos: Optional[Tensor] = None, n_pos: Optional[int] = None) -> Tensor:
         b, n, c = x.shape
         h = self.num_heads
         q, k, v = self.qkv(x).view(b, n, 3, h, c // h).permute(2, 0, 3, 1, 4).unbind(0)
         pos = xpos if self.rope is not None else None
-        q, k = self._norm_rope(q, self.q_norm, pos), self._norm_rope(k, self.k_norm, pos)
+        q, k = self._norm_rope(q, self.q_norm, pos, n_pos), self._norm_rope(k, self.k_norm, pos, n_pos)
         if x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and c // h == 64 and not torch.is_grad_enabled():
             # the package's dense flash kernel (the compressed branch's attention), written straight into [B,N,H,D]
             o = torch.empty((b, n, h, c // h), dtype=x.dtype, device=x.device)
@@ -115,8 +115,8 @@ class Block(nn.Module):
         self.mlp = Mlp(dim, int(dim * mlp_ratio))
         self.ls2 = LayerScale(dim, init_values) if init_values else nn.Identity()
 
-    def forward(self, x: Tensor, xpos: Optional[Tensor] = None) -> Tensor:
-        a = self.attn(token_norm(self.norm1, x), xpos=xpos)
+    def forward(self, x: Tensor, xpos: Optional[Tensor] = None, n_pos: Optional[int] = None) -> Tensor:
+        a = self.attn(token_norm(self.norm1, x), xpos=xpos, n_pos=n_pos)
         x = self.ls1.add_to(x, a) if isinstance(self.ls1, LayerScale) else x + a
         m = self.mlp(token_norm(self.norm2, x))
         return self.ls2.add_to(x, m) if isinstance(self.ls2, LayerScale) else x + m
@@ -165,10 +165,10 @@ class HeadDecoder(nn.Module):
         self.blocks = nn.ModuleList([Block(dim, num_heads, DenseAttentionRope, rope=rope) for _ in range(depth)])
         self.linear_out = nn.Linear(dim, out_dim)
 
-    def forward(self, x: Tensor, xpos: Tensor) -> Tensor:
+    def forward(self, x: Tensor, xpos: Tensor, n_pos: Optional[int] = None) -> Tensor:
         x = self.project(x)
         for blk in self.blocks:
-            x = blk(x, xpos=xpos)
+            x = blk(x, xpos=xpos, n_pos=n_pos)
         return self.linear_out(x)
 
 
@@ -247,9 +247,10 @@ class Pi3SparseLike(nn.Module):
         decoder output the heads read (last frame-local and last global block, concatenated) under "features"."""
         b, f, _, hh, ww = imgs.shape
         gh, gw = hh // self.patch, ww // self.patch
-        # cos/sin tables of the fused norm/RoPE kernel sized for THIS call's grid (patch coordinates run 1..gh, 1..gw;
-        # the kernel clamps positions beyond its table, so a table sized at construction would be wrong for larger frames)
-        self.rope.max_positions = max(gh, gw) + 1
+        # cos/sin tables of the fused norm/RoPE kernels sized for THIS call's grid (patch coordinates run up to gh, gw; the
+        # kernels clamp positions beyond their table, so a table sized at construction would be wrong for larger
+        # frames); handed down call by call, no state shared between calls changes
+        n_pos = max(gh, gw) + 1
         x = ((imgs - self.image_mean) / self.image_std).reshape(b * f, 3, hh, ww).to(self.register_token.dtype)
         x = self.encoder(x)                                                        # [B*F, gh*gw, dim]
         x = torch.cat((self.register_token.expand(b * f, -1, -1), x), dim=1)       # [B*F, T, dim]
@@ -262,16 +263,16 @@ class Pi3SparseLike(nn.Module):
             pos_dec = pos
         local_out = None
         for local_blk, global_blk in zip(self.local_decoder, self.global_decoder):
-            x = local_blk(x, xpos=pos_dec)
+            x = local_blk(x, xpos=pos_dec, n_pos=n_pos)
             local_out = x
-            x = global_blk(x.reshape(b, f * t, -1), xpos=pos_dec.reshape(b, f * t, 2)).reshape(b * f, t, -1)
+            x = global_blk(x.reshape(b, f * t, -1), xpos=pos_dec.reshape(b, f * t, 2), n_pos=n_pos).reshape(b * f, t, -1)
         feat = torch.cat((local_out, x), dim=-1)
         if tiled:                                                                  # the heads see row-major tokens again
             feat = tile_major_inverse(feat, gh, gw, self.tile)
         nreg = self.register_token.shape[1]
-        pts = self.point_head(self.point_decoder(feat, pos)[:, nreg:], gh, gw).float()
-        conf = self.conf_head(self.conf_decoder(feat, pos)[:, nreg:], gh, gw).float()
-        poses = self.camera_head(self.camera_decoder(feat, pos)).reshape(b, f, 4, 4)
+        pts = self.point_head(self.point_decoder(feat, pos, n_pos)[:, nreg:], gh, gw).float()
+        conf = self.conf_head(self.conf_decoder(feat, pos, n_pos)[:, nreg:], gh, gw).float()
+        poses = self.camera_head(self.camera_decoder(feat, pos, n_pos)).reshape(b, f, 4, 4)
         xy, z = pts.split([2, 1], dim=-1)
         z = torch.exp(z)
         local_points = torch.cat((xy * z, z), dim=-1).reshape(b, f, gh * self.patch, gw * self.patch, 3)

@@ -11,6 +11,7 @@ dimension; indices are int32 ``[B, H, n_query_blocks, K]`` in block units.
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -465,6 +466,24 @@ def key_block_lists(idx: torch.Tensor, n_key_blocks: int) -> Tuple[torch.Tensor,
     return lists, off
 
 
+def key_lists_ascending(lists: torch.Tensor, offs: torch.Tensor) -> bool:
+    """Whether every group of ``lists`` ([B,H,L] int32, groups delimited by ``offs`` [B,H,n_key_blocks+1]) is ascending,
+    as :func:`key_block_lists` builds them.  The dK/dV kernel for 16-token blocks merges the lists of four neighbouring
+    key blocks and relies on that order: on a list that is not ascending it skips entries and the gradients come out
+    incomplete WITHOUT an error.  Works on CPU and GPU tensors (on the GPU: a few small kernels and one
+    synchronisation)."""
+    b, h, length = lists.shape
+    if length < 2:
+        return True
+    dev = lists.device
+    starts = torch.zeros((b, h, length + 1), dtype=torch.bool, device=dev)
+    starts.scatter_(2, offs.long().clamp(0, length), True)                      # a pair that straddles a group start is free
+    second = torch.arange(1, length, device=dev)
+    beyond = second >= offs[..., -1:].long()                                     # so is the unspecified tail
+    ok = (lists[..., 1:] >= lists[..., :-1]) | starts[..., 1:length] | beyond
+    return bool(ok.all())
+
+
 def attn_bwd_delta(o: torch.Tensor, dout: torch.Tensor) -> torch.Tensor:
     """``delta[b,h,n] = sum_d o * dout`` in fp32."""
     _need_device(o, dout)
@@ -482,10 +501,13 @@ def attn_bwd_delta(o: torch.Tensor, dout: torch.Tensor) -> torch.Tensor:
 def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
              idx: Optional[torch.Tensor] = None, block: int = 64, softmax_scale: Optional[float] = None,
              need_dq: bool = True, need_dkv: bool = True, delta: Optional[torch.Tensor] = None,
-             key_lists: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+             key_lists: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, check_lists: Optional[bool] = None):
     """Gradients ``(dq, dk, dv)`` of an attention forward with output ``o`` and log-sum-exp ``lse``:
     selection attention over the blocks of ``idx`` ([B,H,Nq_blocks,K] int32), or dense attention (``idx=None``).
-    ``delta`` (:func:`attn_bwd_delta`) and ``key_lists`` (:func:`key_block_lists`) are computed here unless given."""
+    ``delta`` (:func:`attn_bwd_delta`) and ``key_lists`` (:func:`key_block_lists`) are computed here unless given.
+    Caller-built ``key_lists`` must be ascending within every group (see :func:`key_lists_ascending`: with 16-token
+    blocks anything else gives silently incomplete dk, dv); ``check_lists=True`` (default: the environment variable
+    ``S3R_CHECK_LISTS=1``) verifies that here, at the price of a device synchronisation."""
     _need_device(q, k, v, o, dout, lse)
     assert bwd_supported(q, block), "attention backward: built for bf16/fp16, head_dim 64, block 64 or 16"
     q, k, v, o, dout = (_last_contig(t) for t in (q, k, v, o, dout))
@@ -507,6 +529,10 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
         kk = idx.shape[3]
         if need_dkv:
             lists, offs = key_lists if key_lists is not None else key_block_lists(idx, nkb)
+            if key_lists is not None and (check_lists if check_lists is not None else os.environ.get("S3R_CHECK_LISTS") == "1"):
+                if not key_lists_ascending(lists, offs):
+                    raise ValueError("attn_bwd: key_lists must be ascending within every key block's group "
+                                     "(build them with key_block_lists)")
 
     def st(t):
         return (t.stride(0), t.stride(1), t.stride(2)) if t is not None else (0, 0, 0)

@@ -297,3 +297,29 @@ def test_selection_backward_with_blocks_of_128_and_256_tokens(n, block, kk):
     o.backward(g.to(DEV))
     wq, wk, wv = oracle.select_attention_grads_autograd(q, k, v, idx, block, g)
     _close(qd.grad, wq, "dq"); _close(kd.grad, wk, "dk"); _close(vd.grad, wv, "dv")
+
+
+def test_caller_built_lists_that_are_not_ascending_are_refused_on_request():
+    """ops.attn_bwd(check_lists=True): lists from key_block_lists pass; the same lists with one group reversed raise
+    (without the check the 16-token dK/dV kernel would skip entries and return incomplete gradients silently)."""
+    import pytest as _pytest
+    from speed3r_amd.sparse_attn import ops
+    g = torch.Generator().manual_seed(3)
+    n, h, kk, block = 256, 1, 4, 16
+    q, k, v = ((torch.randn((1, h, n, 64), generator=g) * 0.5).to(torch.bfloat16).to("cuda:0") for _ in range(3))
+    nqb = n // block
+    idx = torch.stack([torch.randperm(nqb, generator=g)[:kk] for _ in range(nqb)]).to(torch.int32).view(1, h, nqb, kk).to("cuda:0")
+    o, lse = ops.select_attn(q, k, v, idx, block, return_lse=True)
+    dout = torch.randn(o.shape, generator=g).to(torch.bfloat16).to("cuda:0")
+    lists, offs = ops.key_block_lists(idx, nqb)
+    want = ops.attn_bwd(q, k, v, o, dout, lse, idx, block, key_lists=(lists, offs), check_lists=True)
+    ref = ops.attn_bwd(q, k, v, o, dout, lse, idx, block)
+    assert all(torch.equal(a, b) for a, b in zip(want, ref))
+    lens = (offs[0, 0, 1:] - offs[0, 0, :-1]).cpu()
+    j = int(torch.nonzero(lens >= 2)[0])
+    lo, hi = int(offs[0, 0, j]), int(offs[0, 0, j + 1])
+    bad = lists.clone()
+    bad[0, 0, lo:hi] = lists[0, 0, lo:hi].flip(0)
+    assert not ops.key_lists_ascending(bad, offs)
+    with _pytest.raises(ValueError, match="ascending"):
+        ops.attn_bwd(q, k, v, o, dout, lse, idx, block, key_lists=(bad, offs), check_lists=True)

@@ -150,9 +150,12 @@ def test_layer_gradients_match_autograd_through_the_oracle(n, block_size, topk):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("n,block,with_norm,with_pos", [(320, 64, True, True), (200, 64, True, True), (1041, 16, True, True),
                                                         (77, 16, False, True), (130, 64, True, False), (5, 64, True, True)])
-def test_one_pass_over_the_packed_projection_equals_pooling_then_norm_rope(dtype, n, block, with_norm, with_pos):
+@pytest.mark.parametrize("k_bias", [False, True])
+def test_one_pass_over_the_packed_projection_equals_pooling_then_norm_rope(dtype, n, block, with_norm, with_pos, k_bias):
     """s3r_qkv_prepass (block means of raw q, k, v + LayerNorm + RoPE of q and k in one pass) against s3r_pool_mean on
-    the packed projection followed by s3r_norm_rope on q and k: the same bits, ragged last blocks included."""
+    the packed projection followed by s3r_norm_rope on q and k: the same bits, ragged last blocks included.  With both
+    LayerNorm biases and positions (``k_bias``) the kernel runs the instance the layer module launches, in which norm,
+    biases and rotation are compile-time facts; without the k bias the general one."""
     from speed3r_amd.sparse_attn import ops
     b, h = 2, 3
     g = torch.Generator().manual_seed(n + block)
@@ -161,12 +164,13 @@ def test_one_pass_over_the_packed_projection_equals_pooling_then_norm_rope(dtype
     rope = RoPE2D(freq=100.0)
     cos, sin = rope.tables(64, 40, DEV, dtype) if with_pos else (None, None)
     lnq = ((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV), (0.2 * torch.randn(64, generator=g)).to(dtype).to(DEV))
-    lnk = ((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV), None)
+    lnk = ((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV),
+           (0.2 * torch.randn(64, generator=g)).to(dtype).to(DEV) if k_bias else None)
     got = ops.qkv_prepass(qkv, h, block, pos, cos, sin, lnq if with_norm else None, lnk if with_norm else None, 1e-6)
     q, k, v = qkv.view(b, n, 3, h, 64).permute(2, 0, 3, 1, 4).unbind(0)
     want_c = ops.pool_qkv_packed(qkv, h, block)
     want_q = ops.norm_rope(q, pos, cos, sin, lnq[0] if with_norm else None, lnq[1] if with_norm else None, 1e-6)
-    want_k = ops.norm_rope(k, pos, cos, sin, lnk[0] if with_norm else None, None, 1e-6)
+    want_k = ops.norm_rope(k, pos, cos, sin, lnk[0] if with_norm else None, lnk[1] if with_norm else None, 1e-6)
     assert torch.equal(got[0], want_q) and torch.equal(got[1], want_k)
     assert got[2].data_ptr() == v.data_ptr() and got[2].stride() == v.stride()
     for a, w in zip(got[3:], want_c):

@@ -150,7 +150,7 @@ def test_small_model_in_the_reference_token_order(dtype):
             assert ((g - w).norm() / w.norm()).item() <= 0.02, key
 
 
-def test_rope_tables_follow_the_frame_size():
+def test_rope_tables_follow_the_frame_size(monkeypatch):
     """Frames larger than the grid the model was built for: the fused norm/RoPE kernel's tables are sized from the
     call (positions beyond a table would be clamped): the model's dense attention with RoPE on a 45-wide position range
     against the torch RoPE2D module."""
@@ -169,9 +169,16 @@ def test_rope_tables_follow_the_frame_size():
         want = a.proj((p @ v.float()).to(x.dtype).transpose(1, 2).reshape(1, n, 128))
     assert (got.float() - want.float()).abs().max().item() <= 2e-2
     m = Pi3SparseLike(dim=128, enc_depth=1, dec_depth=2, num_heads=2, head_depth=1, grid=(4, 6), topk=4).to(torch.bfloat16).to(DEV).eval()
+    imgs = torch.rand((1, 2, 3, 14 * 9, 14 * 41), device=DEV)          # 9 x 41 patches on a model built for 4 x 6
+    from speed3r_amd.sparse_attn import ops
+    rows = []
+    real_nr, real_pp = ops.norm_rope, ops.qkv_prepass
+    monkeypatch.setattr(ops, "norm_rope", lambda x, pos, cos, sin, *a, **k: (rows.append(None if cos is None else cos.shape[0]), real_nr(x, pos, cos, sin, *a, **k))[1])
+    monkeypatch.setattr(ops, "qkv_prepass", lambda qkv, h, blk, pos, cos, sin, *a, **k: (rows.append(None if cos is None else cos.shape[0]), real_pp(qkv, h, blk, pos, cos, sin, *a, **k))[1])
     with torch.no_grad():
-        m(torch.rand((1, 2, 3, 14 * 9, 14 * 41), device=DEV))          # 9 x 41 patches on a model built for 4 x 6
-    assert m.rope.max_positions == 42
+        m(imgs)
+    assert rows and all(r in (None, 42) for r in rows) and 42 in rows   # every rotating kernel got a table for coordinates 0..41
+    assert m.rope.max_positions == 8          # as constructed (grid 4 x 6): the call's table size travels with the call
 
 
 def test_end_to_end_workload_100_frames_518x392():
