@@ -33,10 +33,12 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 SETTLE_STEPS = 40           # untimed steps in front of --warmup (clock governor), fixed
-# (config, top-k, block, merge fused) -> HBM bytes per launch of the selection kernel and the profile summary they come from
+# (config, top-k, block, merge fused) -> HBM bytes per launch of the selection kernel, the profile summary they come from
+# and the commit whose kernel was measured (the bytes are a property of the access pattern: list walk, tile size, merge
+# in the epilogue; a change of those makes the figure stale)
 MEASURED_TRAFFIC = {
-    ("cfg3", 16, 64, True): (2.34e9, "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md"),
-    ("cfg4", 16, 64, True): (9.48e9, "profiles/layer_cfg4_1000f_bf16_kernel_stats.md"),
+    ("cfg3", 16, 64, True): (2.34e9, "profiles/select_merge_cfg3_256f_bf16_hbm_bytes.md (kernel of commit 771ade2)"),
+    ("cfg4", 16, 64, True): (9.48e9, "profiles/layer_cfg4_1000f_bf16_kernel_stats.md (kernel of commit e9a5029: same list walk and tiles)"),
 }
 
 

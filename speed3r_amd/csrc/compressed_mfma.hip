@@ -589,9 +589,6 @@ __global__ __launch_bounds__(256, KTOP > 0 ? 3 : 2) void compressed_mfma_kernel(
       }
       thr0 = qvalid ? tau : INFINITY;  // rows beyond Lq (all-zero scores) must not flood the queue
       thr = thr0;
-#ifdef S3R_IDX_NOSURV
-      thr = INFINITY;
-#endif
     }
     // Second sweep: the scores again (same MFMA sequence, same bits), filtered against the threshold; survivors go
     // through the lane's queue into its exact list.
