@@ -147,6 +147,11 @@ int s3r_topk_rows(const float* scores, int32_t* idx, int64_t rows, int cols, int
  *   o:   I/O dtype [B,H,N,D];  lse: optional fp32 [B,H,N] contiguous.
  * Keys beyond N in a partial last block are masked out; a query block with no valid entry
  * gives zeros.  block in {4,16,32,64}, D <= 64 (MFMA paths: block 64 or 16, D == 64, bf16/fp16, K <= 64).
+ * Rounding points of the 64-token MFMA kernel: with lse == NULL the queries are multiplied by
+ * softmax_scale * log2(e) once and rounded to the I/O dtype, and the fp32 scores of those queries are exponents of two
+ * (the reference scales each fp32 score, :100); a query block whose scaled scores leave [-20, 20] (bf16) is recomputed
+ * with the reference's per-score scaling.  With lse != NULL (a forward whose backward will recompute the probabilities
+ * from lse) every score is scaled in fp32 as in the reference.
  * The reference's larger blocks (128, 256; topk_blocksparse_attention.py:862) are the caller's to rewrite, as the
  * Python operator does: the list of a query block serves each of its 64-row parts, a listed key block j becomes the
  * entries r*j .. r*j+r-1 (r = block/64), and the call is made with block 64 and K*r entries per row.
@@ -165,8 +170,10 @@ int s3r_select_attn(const void* q, const void* k, const void* v, const int32_t* 
  * Selection-branch attention with the gated merge in its epilogue: the selection output never
  * goes to memory; the kernel writes
  *   out[b,n,h*D+d] = gate[b,h,n,0]*o_cmp[b,h,n/block,d] + gate[b,h,n,1]*o_sel[b,h,n,d]
- * with the rounding points of s3r_gated_merge (o_sel, each product and the sum rounded to the I/O
- * dtype), so the result equals s3r_select_attn followed by s3r_gated_merge bit for bit.
+ * 16-token blocks: with the rounding points of s3r_gated_merge (o_sel, each product and the sum rounded to the I/O
+ * dtype), so the result equals s3r_select_attn followed by s3r_gated_merge bit for bit.  64-token blocks: the expression
+ * is evaluated in fp32 on the unrounded selection output and rounded ONCE (at most four rounding steps of the I/O dtype,
+ * taken on |gate0 o_cmp| + |gate1 o_sel|, away from the two-call result, on the side of the exact value).
  * Replaces topk_blocksparse_attention (pi3/models/sparse_attn/topk_blocksparse_attention.py:1093-1121)
  * together with the merge expression of pi3/models/layers/sparse_attention.py:127-136.
  * Arguments as in s3r_select_attn and s3r_gated_merge; out is contiguous [B,N,H*D].
