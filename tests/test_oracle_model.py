@@ -32,7 +32,7 @@ def _with_oracle_layers(m):
     for blk in m.global_decoder:
         a = blk.attn
 
-        def fwd(x, attn_bias=None, xpos=None, a=a):
+        def fwd(x, attn_bias=None, xpos=None, n_pos=None, a=a):
             return oracle.sparse_layer(x, a.qkv.weight, a.qkv.bias, a.gate[0].weight, a.gate[0].bias, a.proj.weight, a.proj.bias,
                                        a.num_heads, a.block_size ** 2, a.topk, xpos=xpos, qn_w=a.q_norm.weight,
                                        qn_b=a.q_norm.bias, kn_w=a.k_norm.weight, kn_b=a.k_norm.bias, ln_eps=a.q_norm.eps)["out"]
