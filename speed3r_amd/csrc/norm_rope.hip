@@ -76,9 +76,9 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(
 #pragma unroll
       for (int i = 0; i < VEC; i++) q += (v[i] - mean) * (v[i] - mean);
       q = group_sum<LPR>(q);
-      const float rstd = 1.0f / sqrtf(q * (1.0f / D) + eps);
+      const float rstd = inv_sqrt(q * (1.0f / D) + eps);
 #pragma unroll
-      for (int i = 0; i < VEC; i++) v[i] = round_to<T>((v[i] - mean) * rstd * to_f32(we[i]) + to_f32(be[i]));
+      for (int i = 0; i < VEC; i++) v[i] = round_keep<T>((v[i] - mean) * rstd * to_f32(we[i]) + to_f32(be[i]));
     }
 
     if (pos != nullptr) {  // rotary embedding: the y half turns with pos[...,0], the x half with pos[...,1]
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(
       for (int i = 0; i < VEC; i++) {
         const float other = lane_xor<QL>(v[i]);                 // the paired value, one quarter away
         const float rot = sizeof(T) == 2 || second ? other : -other;  // (16-bit types: the sign is on the sine)
-        const float a = round_to<T>(v[i] * to_f32(ce[i]));
-        const float c2 = round_to<T>(rot * to_f32(se[i]));
+        const float a = round_keep<T>(v[i] * to_f32(ce[i]));
+        const float c2 = round_keep<T>(rot * to_f32(se[i]));
         v[i] = a + c2;
       }
     }

@@ -57,6 +57,19 @@ template <typename T> __device__ __forceinline__ float round_to(float x) {
   return (float)__builtin_bit_cast(T, u);
 }
 template <> __device__ __forceinline__ float round_to<float>(float x) { return x; }
+// The same value for code that goes on in fp32: a bf16 number IS the upper half of its fp32 pattern, so the packed
+// conversion with a zero in the lower half leaves the rounded value ready for use (one instruction per value instead
+// of half a conversion and an unpacking shift or mask).
+template <typename T> __device__ __forceinline__ float round_keep(float x) { return round_to<T>(x); }
+template <> __device__ __forceinline__ float round_keep<bf16_t>(float x) {
+  float r;
+  asm("v_cvt_pk_bf16_f32 %0, 0, %1" : "=v"(r) : "v"(x));
+  return r;
+}
+
+// 1 / sqrt(x) for a normal positive x by the hardware's reciprocal square root (1 ulp): one instruction where
+// sqrtf and the division, both correctly rounded, take about forty.
+__device__ __forceinline__ float inv_sqrt(float x) { return __builtin_amdgcn_rsqf(x); }
 
 // fp32 bit pattern -> order-preserving u32: negative values flip all bits, others the sign bit.
 __device__ __forceinline__ uint32_t sortable_key(float s) {

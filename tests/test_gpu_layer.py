@@ -177,6 +177,30 @@ def test_one_pass_over_the_packed_projection_equals_pooling_then_norm_rope(dtype
         assert a.shape == (b, h, -(-n // block), 64) and torch.equal(a, w)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows", [165, 166, 400])
+def test_one_pass_with_rotation_tables_around_the_lds_limit(dtype, rows):
+    """The layer's instance keeps fp32 copies of the rotation tables in LDS while three tables of ``rows`` x 16 values
+    and the LayerNorm rows fit 32 KB (165 rows do, 166 do not); beyond that it reads the caller's tables as before.
+    Both sides of the limit give the bits of pooling followed by s3r_norm_rope, positions up to the last row included."""
+    from speed3r_amd.sparse_attn import ops
+    b, h, n, block = 1, 2, 700, 64
+    g = torch.Generator().manual_seed(rows)
+    qkv = (torch.randn((b, n, 3 * h * 64), generator=g) * 0.7).to(dtype).to(DEV)
+    pos = torch.randint(0, rows, (b, n, 2), generator=g)
+    pos[0, :4] = torch.tensor([[0, rows - 1], [rows - 1, 0], [rows - 1, rows - 1], [0, 0]])
+    pos = pos.to(DEV)
+    cos, sin = RoPE2D(freq=100.0).tables(64, rows, DEV, dtype)
+    ln = [((1 + 0.3 * torch.randn(64, generator=g)).to(dtype).to(DEV), (0.2 * torch.randn(64, generator=g)).to(dtype).to(DEV))
+          for _ in range(2)]
+    got = ops.qkv_prepass(qkv, h, block, pos, cos, sin, ln[0], ln[1], 1e-6)
+    q, k, v = qkv.view(b, n, 3, h, 64).permute(2, 0, 3, 1, 4).unbind(0)
+    assert torch.equal(got[0], ops.norm_rope(q, pos, cos, sin, ln[0][0], ln[0][1], 1e-6))
+    assert torch.equal(got[1], ops.norm_rope(k, pos, cos, sin, ln[1][0], ln[1][1], 1e-6))
+    for a, w in zip(got[3:], ops.pool_qkv_packed(qkv, h, block)):
+        assert torch.equal(a, w)
+
+
 def test_layer_takes_the_one_pass_route_where_it_is_built():
     torch.manual_seed(11)
     m = SparseFlashAttentionRope(dim=128, num_heads=2, qkv_bias=True, qk_norm=True, rope=RoPE2D(100.0), block_size=8, topk=2)
