@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(
       T* oe = reinterpret_cast<T*>(&out);
 #pragma unroll
       for (int i = 0; i < VEC; i++) oe[i] = from_f32<T>(v[i]);
-      *reinterpret_cast<uint4*>(y + (((int64_t)b * H + h) * N + nn[r]) * D + lr * VEC) = out;
+      store16_nt(y + (((int64_t)b * H + h) * N + nn[r]) * D + lr * VEC, out);
     }
   }
 }

@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void gated_merge_kernel(
     const float c = round_to<T>(g1 * to_f32(es[e]));
     eo[e] = from_f32<T>(a + c);
   }
-  *reinterpret_cast<uint4*>(out + ((int64_t)b * per_batch + i) * VEC) = ro;
+  store16_nt(out + ((int64_t)b * per_batch + i) * VEC, ro);
 }
 
 }  // namespace s3r

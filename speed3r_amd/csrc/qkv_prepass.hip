@@ -217,7 +217,9 @@ __global__ __launch_bounds__(256, 4) void qkv_prepass_kernel(
         uint4 o;
 #pragma unroll
         for (int i = 0; i < VEC; i++) reinterpret_cast<T*>(&o)[i] = from_f32<T>(x[i]);
-        *reinterpret_cast<uint4*>(dst + (t0 + rr) * D) = o;
+        // non-temporal like the loads: nothing of this pass is read again before the attention kernels (0.50 against
+        // 0.55 ms at 266 496 tokens x 16 heads)
+        store16_nt(dst + (t0 + rr) * D, o);
       }
     };
     one(lq, aq, qn_w, qn_b, 0, qo);
