@@ -258,7 +258,8 @@ def _loop_ms(fn, iters=30, settle=20):
 
 def hbm_bound_kernels(qd, kd, vd, gd, block, es):
     """GB/s of the memory-bound kernels, each alone on one stream, from their algorithmic bytes: pooling of one tensor,
-    the layer's one pass over the packed projection, LayerNorm + RoPE of one tensor, the standalone merge."""
+    the layer's one pass over the packed projection, LayerNorm + RoPE of one tensor, the standalone merge; and, for
+    scale, of PyTorch's device-to-device copy of one tensor (``device_copy``: reads and writes 1 : 1, no arithmetic)."""
     import torch
 
     import speed3r_amd as s3r
@@ -289,6 +290,11 @@ def hbm_bound_kernels(qd, kd, vd, gd, block, es):
         ms = _loop_ms(lambda: s3r.gated_merge(o_cmp, vd, gd, block))
         out["merge"] = (2 * n * h * d + n * h * 2 + nc * h * d) * es / (ms * 1e-3) / 1e9
         out["merge_ms"] = ms
+        # for scale: PyTorch's device-to-device copy of one tensor (as many bytes written as read, no arithmetic)
+        buf = torch.empty_like(qd)
+        ms = _loop_ms(lambda: buf.copy_(qd))
+        out["device_copy"] = 2 * n * h * d * es / (ms * 1e-3) / 1e9
+        del buf
     torch.cuda.empty_cache()
     return out
 
