@@ -202,7 +202,9 @@ int s3r_select_attn_merge(const void* q, const void* k, const void* v, const int
  *   cos_tab, sin_tab: I/O dtype [P,16], row p = cos/sin of the angles p * base^(-2i/32), i = 0..15, with the
  *     angles rounded to the I/O dtype first (the reference's table); positions are clamped to [0,P-1].
  *   ln_w, ln_b: I/O dtype [64] LayerNorm weight and bias, ln_w NULL for no normalisation (ln_b optional).
- * Products and sum of the rotation are rounded to the I/O dtype like the reference's eager expression.
+ * Products and sum of the rotation are rounded to the I/O dtype like the reference's eager expression.  The row
+ * statistics are fp32; 1/sqrt(var + eps) comes from the hardware's reciprocal square root (1 ulp), so for 16-bit I/O
+ * a value may land on the neighbouring representable number of the eager result (as it may from the order of the sums).
  */
 int s3r_norm_rope(const void* x, void* y, const int32_t* pos, const void* cos_tab, const void* sin_tab, int P,
                   const void* ln_w, const void* ln_b, float eps,
