@@ -201,6 +201,41 @@ def test_one_pass_with_rotation_tables_around_the_lds_limit(dtype, rows):
         assert torch.equal(a, w)
 
 
+def test_one_pass_at_the_headline_token_count_beyond_4_gib_of_offsets():
+    """266 496 tokens x 16 heads: the packed projection is 1.6 GB, byte offsets of its rows pass 2^31 (64-bit address
+    arithmetic in both routes), the rotated q and k are larger than the last-level cache.  Same bits as pooling followed
+    by s3r_norm_rope; the last rows of the last head are also compared with the torch modules."""
+    from speed3r_amd.sparse_attn import ops
+    b, h, n, block = 1, 16, 266496, 64
+    g = torch.Generator(device=DEV).manual_seed(5)
+    qkv = (torch.randn((b, n, 3 * h * 64), generator=g, device=DEV, dtype=torch.float32) * 0.7).to(torch.bfloat16)
+    t = torch.arange(n, device=DEV) % 1041
+    pos = torch.stack((t // 28, t % 28), dim=-1)[None].contiguous()
+    rope = RoPE2D(freq=100.0)
+    cos, sin = rope.tables(64, 38, DEV, torch.bfloat16)
+    gc = torch.Generator().manual_seed(6)
+    ln = [((1 + 0.3 * torch.randn(64, generator=gc)).to(torch.bfloat16).to(DEV), (0.2 * torch.randn(64, generator=gc)).to(torch.bfloat16).to(DEV))
+          for _ in range(2)]
+    got = ops.qkv_prepass(qkv, h, block, pos, cos, sin, ln[0], ln[1], 1e-6)
+    q, k, v = qkv.view(b, n, 3, h, 64).permute(2, 0, 3, 1, 4).unbind(0)
+    want_q = ops.norm_rope(q, pos, cos, sin, ln[0][0], ln[0][1], 1e-6)
+    assert torch.equal(got[0], want_q)
+    del want_q
+    want_k = ops.norm_rope(k, pos, cos, sin, ln[1][0], ln[1][1], 1e-6)
+    assert torch.equal(got[1], want_k)
+    del want_k
+    for a, w in zip(got[3:], ops.pool_qkv_packed(qkv, h, block)):
+        assert torch.equal(a, w)
+    # the far end against the eager modules (LayerNorm in fp32 on the bf16 values, rounded, then RoPE2D)
+    tail = slice(n - 2082, n)
+    lnq = torch.nn.LayerNorm(64, eps=1e-6).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        lnq.weight.copy_(ln[0][0]); lnq.bias.copy_(ln[0][1])
+        want = rope(lnq(q[:, -1:, tail]).to(torch.bfloat16), pos[:, tail])
+    assert max_abs(got[0][:, -1:, tail], want.float()) <= 4e-2
+    assert (got[0][:, -1:, tail] == want).float().mean().item() >= 0.97
+
+
 def test_layer_takes_the_one_pass_route_where_it_is_built():
     torch.manual_seed(11)
     m = SparseFlashAttentionRope(dim=128, num_heads=2, qkv_bias=True, qk_norm=True, rope=RoPE2D(100.0), block_size=8, topk=2)
