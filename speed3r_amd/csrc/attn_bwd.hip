@@ -696,11 +696,15 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 
   const float scale = p.scale;
   const float sl2 = scale * kLog2e;
-  // bf16: dS = scale * P * (dP - delta) is formed as P * (dP - delta) with the accumulator of dP started at -delta (the
-  // published value) instead of zero, and the softmax scale goes onto dK once at the end: one multiplication per score
-  // instead of a fused multiply-add and a multiplication.  (The rounding of dS to the I/O type is relative, so it does
-  // not care for the factor; fp16, with its narrow range, keeps the scaled value.)  64-token blocks: 2.88 -> 2.79 ms
-  // at 266 496 tokens, top-16.
+  // bf16, 64-token blocks: the per-query terms ride in the accumulators instead of in the vector slots.  The accumulator of
+  // S starts at -lse / scale, so P = exp2(scale * log2(e) * accumulator); the accumulator of dP starts at -delta, so
+  // dS / scale = P * accumulator, and the softmax scale goes onto dK once at the end (the rounding of dS to the I/O type is
+  // relative and does not care for the factor).  Per score that is a multiplication, an exponential and a multiplication
+  // instead of two fused multiply-adds, an exponential and a multiplication, and, what counts more, no LDS read of the
+  // per-query values inside a slot in front of the arithmetic that needs it: the start values come with four
+  // ds_read_b128 per accumulator ahead of the half's products.  2.88 -> 2.79 ms (delta) -> 2.62 ms (lse) at 266 496 tokens,
+  // top-16.  fp16 keeps the scaled dS (narrow range); the 16-token instance has no register to spare (+5 % with it).
+  const float inv_scale = 1.0f / scale;
   constexpr bool FOLD = std::is_same<E, bf16_t>::value && BLK == 64;  // (the 16-token instance has no register to spare: +5 % there)
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
@@ -782,12 +786,13 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     float* const sb = staged_buf == 0 ? lds_s0 : lds_s1;
     if constexpr (BLK == 64) {
       // scaled once here (lse to base 2, delta by the softmax scale) instead of once per score
-      sb[64 * wave + lane] = staged_inf ? INFINITY : wave == 0 ? staged * kLog2e : FOLD ? -staged : staged * scale;
+      if constexpr (FOLD) sb[64 * wave + lane] = staged_inf ? -INFINITY : wave == 0 ? -staged * inv_scale : -staged;
+      else sb[64 * wave + lane] = staged_inf ? INFINITY : staged * (wave == 0 ? kLog2e : scale);
     } else {
       // P of (query, key) counts as often as the key's block lists the query's block: the count goes into the
       // exponent (lse - log2(count); 0 times: lse = +inf), one variant of the query's value per key block
       const bool is_lse = hh == 0;
-      const float base = staged_inf ? INFINITY : is_lse ? staged * kLog2e : FOLD ? -staged : staged * scale;
+      const float base = staged_inf ? INFINITY : staged * (is_lse ? kLog2e : scale);
       const bool plain = __ballot(is_lse && (staged_cnt & 0xfefefefeu) != 0) == 0;  // (wave-uniform) no block listed twice
       float* const to = sb + (is_lse ? 0 : kDeltaAt) + 32 * wave + (lane & 31);
 #pragma unroll
@@ -821,7 +826,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       f32x16 z;
 #pragma unroll
       for (int r = 0; r < 16; r++) z[r] = 0.f;
-      if constexpr (i < 4) sc[HF] = Mma<E>::mma(aq[ks], bk[ks], ks == 0 ? z : sc[HF]);
+      if constexpr (i < 4) sc[HF] = Mma<E>::mma(aq[ks], bk[ks], ks == 0 && !FOLD ? z : sc[HF]);
       else dpv[HF] = Mma<E>::mma(ag[ks], bv[ks], ks == 0 && !FOLD ? z : dpv[HF]);
     };
     // FOLD: the accumulator of a half's dP starts at minus delta of its queries (registers 4g .. 4g+3 hold the queries
@@ -836,6 +841,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
           dpv[HF][4 * g4 + 1] = d4.y;
           dpv[HF][4 * g4 + 2] = d4.z;
           dpv[HF][4 * g4 + 3] = d4.w;
+          const float4 l4 = *reinterpret_cast<const float4*>(sl + 32 * HF + 4 * hh + 8 * g4);
+          sc[HF][4 * g4] = l4.x;
+          sc[HF][4 * g4 + 1] = l4.y;
+          sc[HF][4 * g4 + 2] = l4.z;
+          sc[HF][4 * g4 + 3] = l4.w;
         }
       }
     };
@@ -847,16 +857,18 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     auto vec = [&](auto hf_tag, auto j_tag) {  // scores 2j, 2j+1 of the half: P, dS, both rounded
       constexpr int HF = decltype(hf_tag)::value, j = decltype(j_tag)::value, r = 2 * j;
       // queries 4hh + 8(j/2) + 2(j%2) + {0, 1} of the half
-      const float2 l2 = *reinterpret_cast<const float2*>(sl + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
       f32x16& sh = sc[HF];
       f32x16& dh = dpv[HF];
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(sh[r], sl2, -l2.x));
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(sh[r + 1], sl2, -l2.y));
-      float e0, e1;
+      float p0, p1, e0, e1;
       if constexpr (FOLD) {
+        p0 = __builtin_amdgcn_exp2f(sh[r] * sl2);
+        p1 = __builtin_amdgcn_exp2f(sh[r + 1] * sl2);
         e0 = p0 * dh[r];
         e1 = p1 * dh[r + 1];
       } else {
+        const float2 l2 = *reinterpret_cast<const float2*>(sl + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
+        p0 = __builtin_amdgcn_exp2f(fmaf(sh[r], sl2, -l2.x));
+        p1 = __builtin_amdgcn_exp2f(fmaf(sh[r + 1], sl2, -l2.y));
         const float2 d2 = *reinterpret_cast<const float2*>(sl + kDeltaAt + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
         e0 = p0 * fmaf(dh[r], scale, -d2.x);
         e1 = p1 * fmaf(dh[r + 1], scale, -d2.y);
