@@ -696,16 +696,17 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 
   const float scale = p.scale;
   const float sl2 = scale * kLog2e;
-  // bf16, 64-token blocks: the per-query terms ride in the accumulators instead of in the vector slots.  The accumulator of
-  // S starts at -lse / scale, so P = exp2(scale * log2(e) * accumulator); the accumulator of dP starts at -delta, so
-  // dS / scale = P * accumulator, and the softmax scale goes onto dK once at the end (the rounding of dS to the I/O type is
-  // relative and does not care for the factor).  Per score that is a multiplication, an exponential and a multiplication
-  // instead of two fused multiply-adds, an exponential and a multiplication, and, what counts more, no LDS read of the
-  // per-query values inside a slot in front of the arithmetic that needs it: the start values come with four
-  // ds_read_b128 per accumulator ahead of the half's products.  2.88 -> 2.79 ms (delta) -> 2.62 ms (lse) at 266 496 tokens,
-  // top-16.  fp16 keeps the scaled dS (narrow range); the 16-token instance has no register to spare (+5 % with it).
+  // 64-token blocks: the per-query terms ride in the accumulators instead of in the vector slots.  The accumulator of S
+  // starts at -lse / scale, so P = exp2(scale * log2(e) * accumulator); the accumulator of dP starts at -delta, so
+  // dS / scale = P * accumulator.  No slot then begins with an LDS read of per-query values in front of the arithmetic
+  // that needs them: the start values come with four ds_read_b128 per accumulator ahead of the half's products.  bf16
+  // also puts the softmax scale onto dK once at the end (the rounding of dS to the I/O type is relative and does not care
+  // for the factor): per score a multiplication, an exponential and a multiplication instead of two fused multiply-adds,
+  // an exponential and a multiplication; fp16, with its narrow range, scales every dS.  bf16: 2.88 -> 2.79 ms (delta) ->
+  // 2.62 ms (lse) at 266 496 tokens, top-16.  The 16-token instance has no register to spare (+5 % with it).
   const float inv_scale = 1.0f / scale;
-  constexpr bool FOLD = std::is_same<E, bf16_t>::value && BLK == 64;  // (the 16-token instance has no register to spare: +5 % there)
+  constexpr bool FOLD = BLK == 64;                                   // (the 16-token instance has no register to spare: +5 % there)
+  constexpr bool LATE_SCALE = FOLD && std::is_same<E, bf16_t>::value;  // the softmax scale goes onto dK at the end
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
   const int lse_at = BLK == 16 ? (2 * wave + (c >> 4)) * kVar : 0;
@@ -863,8 +864,8 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       if constexpr (FOLD) {
         p0 = __builtin_amdgcn_exp2f(sh[r] * sl2);
         p1 = __builtin_amdgcn_exp2f(sh[r + 1] * sl2);
-        e0 = p0 * dh[r];
-        e1 = p1 * dh[r + 1];
+        e0 = LATE_SCALE ? p0 * dh[r] : p0 * (dh[r] * scale);
+        e1 = LATE_SCALE ? p1 * dh[r + 1] : p1 * (dh[r + 1] * scale);
       } else {
         const float2 l2 = *reinterpret_cast<const float2*>(sl + 32 * HF + 4 * hh + 8 * (j >> 1) + 2 * (j & 1));
         p0 = __builtin_amdgcn_exp2f(fmaf(sh[r], sl2, -l2.x));
@@ -967,7 +968,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
   E* dvp = (E*)p.dv + (int64_t)b * p.sdvb + (int64_t)h * p.sdvh;
   if constexpr (BLK == 64) {
     walk();
-    if constexpr (FOLD) {
+    if constexpr (LATE_SCALE) {
 #pragma unroll
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -1079,7 +1080,7 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       return true;
     };
     while (build_chunk()) walk();
-    if constexpr (FOLD) {
+    if constexpr (LATE_SCALE) {
 #pragma unroll
       for (int dt = 0; dt < 2; dt++)
 #pragma unroll
