@@ -265,7 +265,8 @@ int s3r_gated_merge(const void* o_cmp, const void* o_sel, const void* gate, void
  * s3r_attn_bwd_delta:  delta[b,h,n] = sum_d o[b,h,n,d] * dout[b,h,n,d]  (fp32, contiguous [B,H,N]).
  * s3r_attn_bwd: with P = exp(scale * q k^T - lse) over the keys the forward attended to,
  *   dv = P^T dout,  dS = scale * P * (dout v^T - delta),  dq = dS k,  dk = dS^T q;
- *   P and dS are rounded to the I/O dtype before the products, accumulation is fp32.
+ *   P and dS are rounded to the I/O dtype before the products, accumulation is fp32 (for dk in bf16 with 64-token
+ *   blocks the rounded factor is dS / scale and the scale multiplies the fp32 sum: the same relative rounding).
  *   lse: the forward's optional output (natural log, scaled scores), fp32 [B,H,Lq] contiguous.
  *   idx: the forward's block indices [B,H,ceil(Lq/block),K] (strides sib,sih,sim), or NULL for dense attention.
  *   kq_list, kq_off (needed for dk/dv when idx is given): for every (b,h) the query-block ids that list key block j,
