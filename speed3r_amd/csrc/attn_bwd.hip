@@ -696,17 +696,19 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
 
   const float scale = p.scale;
   const float sl2 = scale * kLog2e;
-  // 64-token blocks: the per-query terms ride in the accumulators instead of in the vector slots.  The accumulator of S
-  // starts at -lse / scale, so P = exp2(scale * log2(e) * accumulator); the accumulator of dP starts at -delta, so
-  // dS / scale = P * accumulator.  No slot then begins with an LDS read of per-query values in front of the arithmetic
-  // that needs them: the start values come with four ds_read_b128 per accumulator ahead of the half's products.  bf16
-  // also puts the softmax scale onto dK once at the end (the rounding of dS to the I/O type is relative and does not care
-  // for the factor): per score a multiplication, an exponential and a multiplication instead of two fused multiply-adds,
-  // an exponential and a multiplication; fp16, with its narrow range, scales every dS.  bf16: 2.88 -> 2.79 ms (delta) ->
-  // 2.62 ms (lse) at 266 496 tokens, top-16.  The 16-token instance has no register to spare (+5 % with it).
+  // The per-query terms ride in the accumulators instead of in the vector slots.  The accumulator of S starts at
+  // -lse / scale (16-token blocks: the variant of the lane's key block, its count folded in), so P = exp2(scale * log2(e) *
+  // accumulator); the accumulator of dP starts at -delta, so dS / scale = P * accumulator.  No slot then begins with an
+  // LDS read of per-query values in front of the arithmetic that needs them: the start values come with four
+  // ds_read_b128 per accumulator ahead of the half's products (those of the second half's dP a quarter per slot, next
+  // to the fragments of its products: the 16-token instance has no register to spare for all of them at once).  bf16
+  // also puts the softmax scale onto dK once at the end (the rounding of dS to the I/O type is relative and
+  // does not care for the factor): per score a multiplication, an exponential and a multiplication instead of two fused
+  // multiply-adds, an exponential and a multiplication; fp16, with its narrow range, scales every dS.  bf16, 266 496
+  // tokens: 64-token blocks, top-16: 2.88 -> 2.79 (delta) -> 2.62 ms (lse); 16-token blocks, top-32: 3.74 -> 3.67 ms.
   const float inv_scale = 1.0f / scale;
-  constexpr bool FOLD = BLK == 64;                                   // (the 16-token instance has no register to spare: +5 % there)
-  constexpr bool LATE_SCALE = FOLD && std::is_same<E, bf16_t>::value;  // the softmax scale goes onto dK at the end
+  constexpr bool FOLD = true;  // (kept as a switch: the other form reads lse and delta from LDS inside the vector slots)
+  constexpr bool LATE_SCALE = std::is_same<E, bf16_t>::value;  // the softmax scale goes onto dK at the end
   const uint32_t qrow = (uint32_t)p.sqm * (uint32_t)sizeof(E), grow = (uint32_t)p.sgm * (uint32_t)sizeof(E);
   const int tr_off = tr_offset(lane);
   const int lse_at = BLK == 16 ? (2 * wave + (c >> 4)) * kVar : 0;
@@ -793,14 +795,21 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
       // P of (query, key) counts as often as the key's block lists the query's block: the count goes into the
       // exponent (lse - log2(count); 0 times: lse = +inf), one variant of the query's value per key block
       const bool is_lse = hh == 0;
-      const float base = staged_inf ? INFINITY : staged * (is_lse ? kLog2e : scale);
+      const float base = FOLD ? (staged_inf ? -INFINITY : is_lse ? -staged * inv_scale : -staged)
+                              : (staged_inf ? INFINITY : staged * (is_lse ? kLog2e : scale));
       const bool plain = __ballot(is_lse && (staged_cnt & 0xfefefefeu) != 0) == 0;  // (wave-uniform) no block listed twice
       float* const to = sb + (is_lse ? 0 : kDeltaAt) + 32 * wave + (lane & 31);
 #pragma unroll
       for (int kk = 0; kk < 4; kk++) {
         const uint32_t wgt = (staged_cnt >> (8 * kk)) & 0xffu;
-        float vkk = is_lse && wgt == 0 ? INFINITY : base;
-        if (!plain && is_lse) vkk -= __builtin_amdgcn_logf((float)(wgt > 1 ? wgt : 1));
+        float vkk;
+        if constexpr (FOLD) {  // start value of the S accumulator: -(lse - ln(count)) / scale
+          vkk = is_lse && wgt == 0 ? -INFINITY : base;
+          if (!plain && is_lse) vkk += __builtin_amdgcn_logf((float)(wgt > 1 ? wgt : 1)) * (1.0f / sl2);
+        } else {
+          vkk = is_lse && wgt == 0 ? INFINITY : base;
+          if (!plain && is_lse) vkk -= __builtin_amdgcn_logf((float)(wgt > 1 ? wgt : 1));
+        }
         to[kk * kVar] = vkk;
       }
     }
@@ -832,16 +841,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     };
     // FOLD: the accumulator of a half's dP starts at minus delta of its queries (registers 4g .. 4g+3 hold the queries
     // 4hh + 8g .. + 3 of the half)
-    auto delta_init = [&](auto hf_tag) {
+    auto lse_init = [&](auto hf_tag) {
       constexpr int HF = decltype(hf_tag)::value;
       if constexpr (FOLD) {
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
-          const float4 d4 = *reinterpret_cast<const float4*>(sl + kDeltaAt + 32 * HF + 4 * hh + 8 * g4);
-          dpv[HF][4 * g4] = d4.x;
-          dpv[HF][4 * g4 + 1] = d4.y;
-          dpv[HF][4 * g4 + 2] = d4.z;
-          dpv[HF][4 * g4 + 3] = d4.w;
           const float4 l4 = *reinterpret_cast<const float4*>(sl + 32 * HF + 4 * hh + 8 * g4);
           sc[HF][4 * g4] = l4.x;
           sc[HF][4 * g4 + 1] = l4.y;
@@ -849,6 +853,20 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
           sc[HF][4 * g4 + 3] = l4.w;
         }
       }
+    };
+    auto delta_init_piece = [&](auto hf_tag, auto g_tag) {  // registers 4g .. 4g+3 of the half's dP accumulator
+      constexpr int HF = decltype(hf_tag)::value, g4 = decltype(g_tag)::value;
+      if constexpr (FOLD) {
+        const float4 d4 = *reinterpret_cast<const float4*>(sl + kDeltaAt + 32 * HF + 4 * hh + 8 * g4);
+        dpv[HF][4 * g4] = d4.x;
+        dpv[HF][4 * g4 + 1] = d4.y;
+        dpv[HF][4 * g4 + 2] = d4.z;
+        dpv[HF][4 * g4 + 3] = d4.w;
+      }
+    };
+    auto delta_init = [&](auto hf_tag) {
+      lse_init(hf_tag);
+      static_for<4>([&](auto g_tag) { delta_init_piece(hf_tag, g_tag); });
     };
     auto mma_c = [&](auto hf_tag, auto i_tag) {  // product i of 8 of a half's dV^T / dK^T updates
       constexpr int HF = decltype(hf_tag)::value, i = decltype(i_tag)::value, jj = (i >> 1) & 1, dt = i & 1;
@@ -900,10 +918,11 @@ __global__ __launch_bounds__(128, 2) void bwd_dkdv_kernel(BwdParams p, int nkb, 
     // the fragments of a region's second four products are requested four slots ahead, one per slot, so that at most
     // five fragments are in registers at a time
     read_rows<E, true>(qb + kHalfBytes, c, hh, aq);
-    delta_init(H1{});
+    lse_init(H1{});
     static_for<8>([&](auto j_tag) {
       constexpr int j = decltype(j_tag)::value;
       if constexpr (j < 4) ag[j] = read_row_frag<E, true>(gb + kHalfBytes, c, hh, j);
+      if constexpr (j < 4) delta_init_piece(H1{}, j_tag);  // (a quarter per slot: needed from the fifth product on)
       mma_a(H1{}, j_tag);
       vec(H0{}, j_tag);
       __builtin_amdgcn_sched_barrier(0);
